@@ -1,0 +1,81 @@
+"""Device tensors behind the cache manager's pages and slots.
+
+Per cache group one K pool ``[n_layers, n_pages, KV, P, hd]`` and one V pool
+``[n_layers, n_pages, KV, hd, P]``: a page of one layer's keys is ``P`` rows of
+``hd`` contiguous elements per head; a page of values is stored transposed so
+that the keys of a page are contiguous for one head dimension.  (The
+reference keeps per layer ``[n_pages*P, KV, hd]`` for both,
+``fastgen/cache.py:66-78``.)  Pages are not cleared when they change hands:
+what a page holds beyond a request's length is never read.
+
+Per-request state of fixed size lives in ``[n_slots, *shape]`` tensors, one
+per run entry that asked for it, cleared when a slot is handed out.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import LayerStore, PagedNeed, StateNeed
+
+
+@dataclass(frozen=True)
+class CacheGroup:
+    need: PagedNeed
+    entries: Tuple[int, ...]  # run-order indices that own pages in this group
+
+
+def group_entries(needs: Sequence[Optional[PagedNeed]]) -> List[CacheGroup]:
+    """Run entries with equal needs share a group (and so a block table)."""
+    by_need: Dict[PagedNeed, List[int]] = {}
+    for i, n in enumerate(needs):
+        if n is not None:
+            by_need.setdefault(n, []).append(i)
+    return [CacheGroup(n, tuple(e)) for n, e in by_need.items()]
+
+
+class CacheStorage:
+    def __init__(self, groups: Sequence[CacheGroup], pages_per_group: Sequence[int], page_size: int,
+                 state_needs: Dict[int, StateNeed], n_slots: int, dtype: torch.dtype,
+                 device: torch.device | str) -> None:
+        self.groups = list(groups)
+        self.page_size = page_size
+        self.k: List[torch.Tensor] = []
+        self.v: List[torch.Tensor] = []
+        self._where: Dict[int, Tuple[int, int]] = {}  # run entry -> (group, layer index in group)
+        for g, (grp, n_pages) in enumerate(zip(self.groups, pages_per_group)):
+            kv, hd = grp.need.n_kv_heads, grp.need.head_dim
+            n = len(grp.entries)
+            self.k.append(torch.empty((n, n_pages, kv, page_size, hd), dtype=dtype, device=device))
+            self.v.append(torch.empty((n, n_pages, kv, hd, page_size), dtype=dtype, device=device))
+            for j, e in enumerate(grp.entries):
+                self._where[e] = (g, j)
+        self.state: Dict[int, torch.Tensor] = {
+            e: torch.zeros((n_slots, *need.shape), dtype=need.dtype, device=device)
+            for e, need in state_needs.items()
+        }
+
+    def store_for(self, entry: int, owner: Optional[int] = None) -> LayerStore:
+        """Storage of run entry ``entry``; with ``owner`` the storage of that
+        earlier entry, read only."""
+        src = entry if owner is None else owner
+        st = LayerStore(owns=owner is None)
+        if src in self._where:
+            g, j = self._where[src]
+            st.group, st.k_pages, st.v_pages = g, self.k[g][j], self.v[g][j]
+        st.state = self.state.get(src)
+        return st
+
+    def reset_slot(self, slot: int) -> None:
+        for t in self.state.values():
+            t[slot].zero_()
+
+    def bytes_per_token(self) -> int:
+        """Cache bytes one token takes over all layers (``fastgen/cache.py`` ``bytes_per_token``)."""
+        return sum(
+            2 * len(g.entries) * g.need.n_kv_heads * g.need.head_dim * self.k[i].element_size()
+            for i, g in enumerate(self.groups)
+        )

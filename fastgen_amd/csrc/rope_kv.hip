@@ -1,0 +1,91 @@
+// Rotary position encoding of q and k and the write of k, v into the paged
+// cache, in one launch (the reference issues four: fastgen/forward.py:449-460
+// with kernels/rope.py and kernels/paged_memcpy.py).
+//
+// Rotation (kernels/rope.py:56-89): pair (x[2i], x[2i+1]) of a head, angle =
+// float(pos) * freqs[i] in fp32, precise sin/cos,
+//   x[2i] = a cos - b sin,  x[2i+1] = b cos + a sin,
+// rounded once at the store.  Pairs beyond rotary_dim are left as they are.
+//
+// Cache layout, per cache layer: K pages [n_pages, KV, P, hd] (a key's head
+// is hd contiguous elements), V pages [n_pages, KV, hd, P] (transposed: the
+// keys of a page are contiguous for one head dimension), so that both matrix
+// products of attention read 16 contiguous bytes per lane.  A token's place
+// is slot = page*P + offset; a negative slot means "write nothing".
+#include "common.h"
+
+#define ROPE_THREADS 256
+
+template <class T>
+__global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
+    T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+    const float* __restrict__ freqs, const int* __restrict__ slots, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
+    int write_kv) {
+  const int t = blockIdx.x;
+  T* row = qkv + (size_t)t * row_stride;
+  const float pos = (float)positions[t];
+  const int half = hd / 2;
+  const int slot = write_kv ? slots[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+
+  // q heads then k heads: (n_heads + n_kv) * hd/2 pairs
+  const int n_rot_heads = n_heads + (write_kv ? n_kv : 0);
+  const int n_pairs = n_rot_heads * half;
+  for (int p = threadIdx.x; p < n_pairs; p += ROPE_THREADS) {
+    const int head = p / half, i = p % half;
+    T* x = row + (size_t)head * hd + 2 * i;
+    float a = to_f<T>(x[0]), b = to_f<T>(x[1]);
+    if (2 * i < rotary_dim) {
+      const float ang = pos * freqs[i];
+      const float s = sinf(ang), c = cosf(ang);
+      const float ra = a * c - b * s;
+      const float rb = b * c + a * s;
+      a = ra;
+      b = rb;
+    }
+    if (head < n_heads) {
+      x[0] = from_f<T>(a);
+      x[1] = from_f<T>(b);
+    } else if (slot >= 0) {
+      const int kvh = head - n_heads;
+      T* dst = k_pages + (((size_t)page * n_kv + kvh) * page_size + off) * hd + 2 * i;
+      dst[0] = from_f<T>(a);
+      dst[1] = from_f<T>(b);
+    }
+  }
+  if (slot >= 0) {
+    const T* v = row + (size_t)(n_heads + n_kv) * hd;
+    for (int e = threadIdx.x; e < n_kv * hd; e += ROPE_THREADS) {
+      const int kvh = e / hd, d = e % hd;
+      v_pages[(((size_t)page * n_kv + kvh) * hd + d) * page_size + off] = v[e];
+    }
+  }
+}
+
+// qkv: [n_tokens, row_stride] with q heads, then k heads, then v heads in a
+// row.  With write_kv == 0 only q is rotated (a mixer that reads another
+// layer's cache).
+extern "C" int fg_rope_kv_write(void* qkv, int row_stride, const int* positions,
+                                const float* freqs, const int* slots, void* k_pages,
+                                void* v_pages, int n_tokens, int n_heads, int n_kv, int hd,
+                                int rotary_dim, int page_size, int write_kv, int dtype,
+                                hipStream_t stream) {
+  if (n_tokens <= 0) return FG_OK;
+  if (hd <= 0 || hd % 2 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 ||
+      page_size <= 0 || n_heads <= 0 || n_kv < 0)
+    return FG_ERR_ARG;
+  if (row_stride < (n_heads + (write_kv ? 2 * n_kv : 0)) * hd) return FG_ERR_ARG;
+  if (dtype == FG_F32)
+    rope_kv_write_kernel<float><<<n_tokens, ROPE_THREADS, 0, stream>>>(
+        (float*)qkv, row_stride, positions, freqs, slots, (float*)k_pages, (float*)v_pages,
+        n_heads, n_kv, hd, rotary_dim, page_size, write_kv);
+  else if (dtype == FG_BF16)
+    rope_kv_write_kernel<bf16_t><<<n_tokens, ROPE_THREADS, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, positions, freqs, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
+        n_heads, n_kv, hd, rotary_dim, page_size, write_kv);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}

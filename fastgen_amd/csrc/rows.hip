@@ -1,0 +1,161 @@
+// Row-wise kernels: embedding gather, residual add fused with RMSNorm,
+// SiLU(gate)*up.  The residual stream is fp32 in both precisions.
+//
+// Formulas: embedding fastgen/forward.py:406-409; RMSNorm
+// fastgen/kernels/rmsnorm.py:33-60 (fp32 sum of squares, rsqrt(mean+eps),
+// a*rstd*w left to right, one rounding at the store); SiLU*mul
+// fastgen/forward.py:495 (here in fp32 with one rounding).
+#include "common.h"
+
+#define ROWS_THREADS 256
+
+// ---------------------------------------------------------------- embedding
+template <class TW>
+__global__ __launch_bounds__(ROWS_THREADS) void embed_kernel(
+    const TW* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ out,
+    int dim, int vocab) {
+  const int t = blockIdx.x;
+  int tok = tokens[t];
+  // ids are validated on the host; the clamp only keeps a bad id from faulting
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  const TW* src = table + (size_t)tok * dim;
+  float* dst = out + (size_t)t * dim;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) dst[i] = to_f<TW>(src[i]);
+}
+
+extern "C" int fg_embed(const void* table, int table_dtype, const int* tokens, float* out,
+                        int n_tokens, int dim, int vocab, hipStream_t stream) {
+  if (n_tokens <= 0) return FG_OK;
+  if (dim <= 0 || vocab <= 0) return FG_ERR_ARG;
+  if (table_dtype == FG_F32)
+    embed_kernel<float><<<n_tokens, ROWS_THREADS, 0, stream>>>((const float*)table, tokens, out, dim, vocab);
+  else if (table_dtype == FG_BF16)
+    embed_kernel<bf16_t><<<n_tokens, ROWS_THREADS, 0, stream>>>((const bf16_t*)table, tokens, out, dim, vocab);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------ residual add + norm
+// Row r of the output is norm(h[src] (+ delta[src])) * w with src = rows ?
+// rows[r] : r.  When delta is given and all rows are normed (rows == null)
+// the sum is written back to h, so the residual stream is updated in the pass
+// that reads it for the norm; a gathered call leaves h as it is (rows may
+// name a row twice).
+template <class TA, class TW>
+__global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_kernel(
+    float* __restrict__ h, const TA* __restrict__ delta, const TW* __restrict__ w,
+    TA* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* hrow = h + src * dim;
+  const TA* drow = delta ? delta + src * dim : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
+    float v = hrow[i];
+    if (drow) {
+      v += to_f<TA>(drow[i]);
+      if (!rows) hrow[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss / (float)dim + eps);
+  TA* orow = out + (size_t)r * dim;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
+    // each thread re-reads only what it wrote itself above
+    float v = hrow[i];
+    if (drow && rows) v += to_f<TA>(drow[i]);
+    orow[i] = from_f<TA>(v * rstd * to_f<TW>(w[i]));
+  }
+}
+
+extern "C" int fg_add_rmsnorm(float* h, const void* delta, const void* w, void* out,
+                              const int* rows, int n_rows, int dim, float eps, int act_dtype,
+                              int w_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (dim <= 0) return FG_ERR_ARG;
+#define LAUNCH(TA, TW)                                                                       \
+  add_rmsnorm_kernel<TA, TW><<<n_rows, ROWS_THREADS, 0, stream>>>(                           \
+      h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps)
+  if (act_dtype == FG_F32 && w_dtype == FG_F32) LAUNCH(float, float);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_F32) LAUNCH(bf16_t, float);
+  else if (act_dtype == FG_F32 && w_dtype == FG_BF16) LAUNCH(float, bf16_t);
+  else return FG_ERR_ARG;
+#undef LAUNCH
+  return fg_launch_status();
+}
+
+// Plain RMSNorm over rows of act dtype (no residual), for norms that sit
+// elsewhere than on the residual stream (per head, after a block).
+template <class TA, class TW>
+__global__ __launch_bounds__(ROWS_THREADS) void rmsnorm_kernel(
+    const TA* __restrict__ x, const TW* __restrict__ w, TA* __restrict__ out, int dim,
+    float eps) {
+  __shared__ float red[16];
+  const TA* xrow = x + (size_t)blockIdx.x * dim;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
+    float v = to_f<TA>(xrow[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss / (float)dim + eps);
+  TA* orow = out + (size_t)blockIdx.x * dim;
+  for (int i = threadIdx.x; i < dim; i += ROWS_THREADS)
+    orow[i] = from_f<TA>(to_f<TA>(xrow[i]) * rstd * to_f<TW>(w[i]));
+}
+
+extern "C" int fg_rmsnorm(const void* x, const void* w, void* out, int n_rows, int dim,
+                          float eps, int act_dtype, int w_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (dim <= 0) return FG_ERR_ARG;
+#define LAUNCH(TA, TW)                                                                       \
+  rmsnorm_kernel<TA, TW><<<n_rows, ROWS_THREADS, 0, stream>>>((const TA*)x, (const TW*)w,    \
+                                                              (TA*)out, dim, eps)
+  if (act_dtype == FG_F32 && w_dtype == FG_F32) LAUNCH(float, float);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (act_dtype == FG_BF16 && w_dtype == FG_F32) LAUNCH(bf16_t, float);
+  else if (act_dtype == FG_F32 && w_dtype == FG_BF16) LAUNCH(float, bf16_t);
+  else return FG_ERR_ARG;
+#undef LAUNCH
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------------- SiLU(g) * u
+// gu is [n_rows, 2*hidden]: the gate columns first, then the up columns.
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void silu_mul_kernel(
+    const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
+  const TA* g = gu + (size_t)blockIdx.y * 2 * hidden;
+  const TA* u = g + hidden;
+  TA* o = out + (size_t)blockIdx.y * hidden;
+  const int i = blockIdx.x * ROWS_THREADS + threadIdx.x;
+  if (i < hidden) {
+    const float gv = to_f<TA>(g[i]);
+    const float uv = to_f<TA>(u[i]);
+    o[i] = from_f<TA>(gv / (1.f + expf(-gv)) * uv);
+  }
+}
+
+extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, int act_dtype,
+                           hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (hidden <= 0 || n_rows > 65535 * 32) return FG_ERR_ARG;
+  // blockIdx.y is limited to 65535: rows beyond that go to further launches
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    dim3 grid((hidden + ROWS_THREADS - 1) / ROWS_THREADS, nr);
+    if (act_dtype == FG_F32)
+      silu_mul_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(
+          (const float*)gu + (size_t)r0 * 2 * hidden, (float*)out + (size_t)r0 * hidden, hidden);
+    else if (act_dtype == FG_BF16)
+      silu_mul_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(
+          (const bf16_t*)gu + (size_t)r0 * 2 * hidden, (bf16_t*)out + (size_t)r0 * hidden, hidden);
+    else
+      return FG_ERR_ARG;
+  }
+  return fg_launch_status();
+}

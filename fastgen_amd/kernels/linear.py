@@ -1,0 +1,50 @@
+"""``y = x W^T`` for the two precisions of the engine.
+
+float32: the engine's own fused-multiply-add kernel (``gemm.hip``), a true
+32-bit product whose rows do not depend on one another.  bfloat16: the
+vendor library's matrix product through ``torch`` (the reference uses cuBLAS
+through ``F.linear`` for the same products, ``fastgen/forward.py:433-513``),
+with fp32 accumulation; logits are asked for in fp32 directly.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import ops
+
+_mm_out_dtype_ok: Optional[bool] = None
+
+
+def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+    """bf16 x bf16 -> fp32 through the library if this torch build offers it."""
+    global _mm_out_dtype_ok
+    if _mm_out_dtype_ok is False:
+        return None
+    try:
+        y = torch.mm(x, w.t(), out_dtype=torch.float32)
+        _mm_out_dtype_ok = True
+        return y
+    except (TypeError, RuntimeError):
+        if _mm_out_dtype_ok is None:
+            _mm_out_dtype_ok = False
+            return None
+        raise
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    if not x.is_cuda:
+        raise ops.KernelArgumentError("fastgen_amd runs on the GPU only; got a tensor on " + str(x.device))
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise ops.KernelArgumentError("a float32 product has float32 output")
+        return ops.gemm_nt(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
+    if out_dtype == torch.bfloat16:
+        return torch.nn.functional.linear(x, w)
+    y = _library_mm_f32_out(x, w)
+    return y if y is not None else ops.gemm_nt(x, w, out_dtype=torch.float32)

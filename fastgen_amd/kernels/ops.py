@@ -1,0 +1,283 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that the operands have the shapes, dtypes
+and strides the kernel and its grid assume, then launches on the current
+stream of the tensors' device.  Nothing here runs on the CPU: a tensor that
+is not on a GPU is refused.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelArgumentError(ValueError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelArgumentError(f"dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelArgumentError(msg)
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _need(t.is_cuda, "fastgen_amd kernels run on the GPU only; got a tensor on " + str(t.device))
+        dev = dev or t.device
+        _need(t.device == dev, "operands live on different devices")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _check(status: int, what: str) -> None:
+    if status == 1:
+        raise KernelArgumentError(f"{what}: the kernel refuses these sizes or dtypes")
+    if status != 0:
+        raise RuntimeError(f"{what}: launch failed (status {status})")
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+    if n is not None:
+        _need(t.numel() >= n, f"{name} holds {t.numel()} entries, {n} are needed")
+
+
+# --------------------------------------------------------------------- rows
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[tokens[t]] as fp32 (``fastgen/forward.py:406-409``)."""
+    _gpu(table, tokens, out)
+    n = tokens.numel()
+    _need(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [vocab, dim]")
+    _i32(tokens, "tokens")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (n, table.shape[1]),
+          "out must be contiguous float32 [n_tokens, dim]")
+    st = _lib.load("rows").fg_embed(
+        _ptr(table), _code(table), _ptr(tokens), _ptr(out), n, table.shape[1], table.shape[0], _stream(out))
+    _check(st, "embed")
+    return out
+
+
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``h += delta`` (fp32 residual stream), ``out = rmsnorm(h) * weight``.
+
+    With ``rows`` only those rows of ``h`` are normed, into consecutive rows
+    of ``out``, and ``h`` is left unchanged.  Norm as in
+    ``fastgen/kernels/rmsnorm.py:33-60``.
+    """
+    _gpu(h, delta, weight, out, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [T, dim]")
+    T, dim = h.shape
+    n_rows = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, "rows")
+    _need(weight.shape == (dim,) and weight.is_contiguous(), "weight must be [dim]")
+    _need(out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
+    if delta is not None:
+        _need(delta.shape == h.shape and delta.is_contiguous() and delta.dtype == out.dtype,
+              "delta must be contiguous, shaped like h, of out's dtype")
+    st = _lib.load("rows").fg_add_rmsnorm(
+        _ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), n_rows, dim, ctypes.c_float(eps),
+        _code(out), _code(weight), _stream(out))
+    _check(st, "add_rmsnorm")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm over the last dimension of a contiguous tensor."""
+    _gpu(x, weight, out)
+    _need(x.is_contiguous(), "x must be contiguous")
+    dim = x.shape[-1]
+    out = torch.empty_like(x) if out is None else out
+    _need(out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous(), "out must match x")
+    _need(weight.shape == (dim,) and weight.is_contiguous(), "weight must be [dim]")
+    st = _lib.load("rows").fg_rmsnorm(
+        _ptr(x), _ptr(weight), _ptr(out), x.numel() // dim, dim, ctypes.c_float(eps), _code(x),
+        _code(weight), _stream(out))
+    _check(st, "rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` of ``[T, 2*hidden]`` (gate columns first), fp32 inside."""
+    _gpu(gate_up, out)
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
+          "gate_up must be contiguous [T, 2*hidden]")
+    T, hidden = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, hidden), dtype=gate_up.dtype, device=gate_up.device) if out is None else out
+    _need(out.shape == (T, hidden) and out.dtype == gate_up.dtype and out.is_contiguous(), "out must be [T, hidden]")
+    st = _lib.load("rows").fg_silu_mul(_ptr(gate_up), _ptr(out), T, hidden, _code(out), _stream(out))
+    _check(st, "silu_mul")
+    return out
+
+
+# ------------------------------------------------------------ rope + kv write
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[torch.Tensor],
+                  slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                  v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
+                  rotary_dim: int, write_kv: bool = True) -> None:
+    """Rotate q and k of ``qkv [T, (H+2KV)*hd]`` in place and store k, v at
+    ``slots`` of the paged cache (K pages ``[n_pages, KV, P, hd]``, V pages
+    ``[n_pages, KV, hd, P]``).  ``kernels/rope.py:56-89``, ``forward.py:449-460``.
+    """
+    _gpu(qkv, positions, freqs, slots, k_pages, v_pages)
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qkv must be [T, width] with unit column stride")
+    T = qkv.shape[0]
+    width = (n_heads + (2 * n_kv if write_kv else 0)) * head_dim
+    _need(qkv.shape[1] >= width, f"qkv rows hold {qkv.shape[1]} elements, {width} are needed")
+    _i32(positions, "positions", T)
+    _need(head_dim % 2 == 0 and 0 <= rotary_dim <= head_dim and rotary_dim % 2 == 0,
+          "head_dim and rotary_dim must be even and rotary_dim <= head_dim")
+    if rotary_dim:
+        _need(freqs is not None and freqs.dtype == torch.float32 and freqs.is_contiguous()
+              and freqs.numel() >= rotary_dim // 2, "freqs must be float32 [rotary_dim/2]")
+    page_size = 1
+    if write_kv:
+        _need(slots is not None and k_pages is not None and v_pages is not None, "cache operands missing")
+        _i32(slots, "slots", T)
+        _need(k_pages.dim() == 4 and k_pages.is_contiguous() and k_pages.dtype == qkv.dtype
+              and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim,
+              "k_pages must be contiguous [n_pages, KV, P, hd] of qkv's dtype")
+        page_size = k_pages.shape[2]
+        _need(v_pages.is_contiguous() and v_pages.dtype == qkv.dtype
+              and v_pages.shape == (k_pages.shape[0], n_kv, head_dim, page_size),
+              "v_pages must be contiguous [n_pages, KV, hd, P] of qkv's dtype")
+    st = _lib.load("rope_kv").fg_rope_kv_write(
+        _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(freqs), _ptr(slots), _ptr(k_pages), _ptr(v_pages),
+        T, n_heads, n_kv, head_dim, rotary_dim, page_size, int(write_kv), _code(qkv), _stream(qkv))
+    _check(st, "rope_kv_write")
+
+
+# ------------------------------------------------------------------ attention
+def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                            block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
+                            n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Causal attention of every token over its sequence's cached keys.
+
+    ``q`` is ``[T, >= H*hd]`` (the first ``H*hd`` columns are the query heads;
+    it may be a qkv buffer), ``out`` is ``[T, H*hd]``.  ``forward.py:176-258``.
+    """
+    _gpu(q, out, k_pages, v_pages, block_table, seq_of_token, positions)
+    T = q.shape[0]
+    _need(k_pages.dim() == 4 and k_pages.is_contiguous(), "k_pages must be contiguous [n_pages, KV, P, hd]")
+    n_pages, n_kv, page_size, hd = k_pages.shape
+    _need(v_pages.shape == (n_pages, n_kv, hd, page_size) and v_pages.is_contiguous(),
+          "v_pages must be contiguous [n_pages, KV, hd, P]")
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * hd, "q must be [T, >= H*hd]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape == (T, n_heads * hd), "out must be [T, H*hd]")
+    _need(q.dtype == out.dtype == k_pages.dtype == v_pages.dtype, "q, out and the cache must share a dtype")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, max_pages]")
+    _i32(seq_of_token, "seq_of_token", T)
+    _i32(positions, "positions", T)
+    _need(n_heads % n_kv == 0, "the number of heads must be a multiple of the number of kv heads")
+    _need(hd % 8 == 0 and hd <= 512, f"head size {hd} is not supported (multiple of 8, at most 512)")
+    _need(page_size % 8 == 0, f"page size {page_size} is not supported (multiple of 8)")
+    st = _lib.load("attention").fg_paged_attention_general(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+        block_table.stride(0), _ptr(seq_of_token), _ptr(positions), T, n_heads, n_kv, hd, page_size,
+        ctypes.c_float(scale), int(window or 0), _code(q), _stream(q))
+    _check(st, "paged_attention_general")
+    return out
+
+
+def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                    group, ctx, n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Attention for one step: picks the kernel for the step's shape.
+
+    ``group`` carries the block table of the layer's cache group, ``ctx`` the
+    step's per-token vectors (``fastgen_amd.engine.context``).
+    """
+    return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token,
+                                   ctx.positions, n_heads, scale, window)
+
+
+# ----------------------------------------------------------------------- gemm
+def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x @ w.T`` with ``w [N, K]``, by the engine's own fp32-FMA kernel (sum
+    over k in ascending order; a row's result does not depend on the others)."""
+    _gpu(x, w, out)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
+    _need(x.stride(1) == 1 and w.stride(1) == 1, "x and w need unit column stride")
+    _need(x.dtype == w.dtype, "x and w must share a dtype")
+    M, K = x.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
+    _need(out.shape == (M, N) and out.stride(1) == 1, "out must be [M, N]")
+    for m0 in range(0, M, 65535 * 64):  # grid.y limit
+        m1 = min(M, m0 + 65535 * 64)
+        st = _lib.load("gemm").fg_gemm_nt(
+            _ptr(x[m0:m1]), _ptr(w), _ptr(out[m0:m1]), m1 - m0, N, K, x.stride(0), w.stride(0), out.stride(0),
+            _code(x), _code(out), _stream(out))
+        _check(st, "gemm_nt")
+    return out
+
+
+# ------------------------------------------------------------------- sampling
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           top_p: Optional[torch.Tensor] = None, seeds: Optional[torch.Tensor] = None,
+           counters: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token id per row of fp32 ``logits [n, V]``: argmax where the row's
+    temperature is 0 (or none is given), else a draw from
+    ``softmax(logits / temperature)`` cut to the ``top_p`` nucleus, with the
+    uniform number taken from ``(seeds[row], counters[row])``.
+    ``fastgen/generate.py:887-896``, ``utils/sampling.py:6-31``.
+    """
+    _gpu(logits, temperature, top_p, seeds, counters, out)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
+          "logits must be float32 [n, V]")
+    n, V = logits.shape
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device) if out is None else out
+    _i32(out, "out", n)
+    for name, t in (("temperature", temperature), ("top_p", top_p)):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n, f"{name} must be float32 [n]")
+    for name, t in (("seeds", seeds), ("counters", counters)):
+        if t is not None:
+            _need(t.dtype == torch.int64 and t.is_contiguous() and t.numel() >= n, f"{name} must be int64 [n]")
+    if temperature is not None:
+        _need(seeds is not None and counters is not None, "sampling needs seeds and counters")
+    st = _lib.load("sampling").fg_sample(
+        _ptr(logits), logits.stride(0), n, V, _ptr(temperature), _ptr(top_p), _ptr(seeds), _ptr(counters),
+        _ptr(out), _stream(logits))
+    _check(st, "sample")
+    return out
+
+
+def logprob(logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+    """``log_softmax(logits)[row, tokens[row]]`` (``fastgen/generate.py:725-730``)."""
+    _gpu(logits, tokens)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
+          "logits must be float32 [n, V]")
+    n, V = logits.shape
+    _i32(tokens, "tokens", n)
+    out = torch.empty((n,), dtype=torch.float32, device=logits.device)
+    st = _lib.load("sampling").fg_logprob(_ptr(logits), logits.stride(0), n, V, _ptr(tokens), _ptr(out), _stream(logits))
+    _check(st, "logprob")
+    return out

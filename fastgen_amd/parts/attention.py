@@ -1,0 +1,74 @@
+"""Grouped-query causal attention over the paged cache.
+
+Per step (``fastgen/forward.py:421-472``): one product for q, k and v (the
+three projections are stored as one matrix), rotation of q and k and the
+write of k, v into the pages in one launch, attention of every new token
+over all cached keys of its request, output projection.
+"""
+
+from __future__ import annotations
+
+from typing import Any, List, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from ..kernels.linear import linear
+from .base import LayerStore, Mixer, PagedNeed, TensorSpec, build_part, place, register_part, MATRIX
+
+
+class Attention(Mixer):
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        o = spec.options
+        self.dim = int(o["dim"])
+        self.n_heads = int(o["n_heads"])
+        self.n_kv_heads = int(o["n_kv_heads"])
+        self.head_dim = int(o["head_dim"])
+        self.scale = float(o.get("scale", self.head_dim**-0.5))
+        self.window: Optional[int] = o.get("window") or None
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError(f"n_heads={self.n_heads} is not a multiple of n_kv_heads={self.n_kv_heads}")
+        self.position = build_part("position", o["position"])
+        self.wqkv: Optional[torch.Tensor] = None
+        self.wo: Optional[torch.Tensor] = None
+        self.freqs: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        q, kv = self.n_heads * self.head_dim, self.n_kv_heads * self.head_dim
+        return [
+            TensorSpec(self._name("q_proj.weight"), (q, self.dim)),
+            TensorSpec(self._name("k_proj.weight"), (kv, self.dim)),
+            TensorSpec(self._name("v_proj.weight"), (kv, self.dim)),
+            TensorSpec(self._name("o_proj.weight"), (self.dim, q)),
+        ]
+
+    def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
+        wq = self.position.arrange_rows(tensors[self._name("q_proj.weight")], self.n_heads)
+        wk = self.position.arrange_rows(tensors[self._name("k_proj.weight")], self.n_kv_heads)
+        wv = tensors[self._name("v_proj.weight")]
+        self.wqkv = place(torch.cat([wq, wk, wv], dim=0), MATRIX, dtype, device)
+        self.wo = place(tensors[self._name("o_proj.weight")], MATRIX, dtype, device)
+        f = self.position.frequencies()
+        self.freqs = None if f is None else f.to(device=device, dtype=torch.float32).contiguous()
+
+    def paged_need(self) -> PagedNeed:
+        return PagedNeed(self.n_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x: torch.Tensor, ctx: Any, store: LayerStore) -> torch.Tensor:
+        group = ctx.groups[store.group]
+        q_width = self.n_heads * self.head_dim
+        # an entry that reads another entry's cache needs its queries only
+        w = self.wqkv if store.owns else self.wqkv[:q_width]
+        qkv = linear(x, w)
+        ops.rope_kv_write(
+            qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
+            self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
+        )
+        out = torch.empty((x.shape[0], q_width), dtype=x.dtype, device=x.device)
+        ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,
+                            self.window or 0)
+        return linear(out, self.wo)
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,40 @@
+"""Dense gated feed-forward (``fastgen/forward.py:483-499``):
+``down(silu(gate(x)) * up(x))``.  Gate and up are one matrix, so one product
+gives both."""
+
+from __future__ import annotations
+
+from typing import Any, List, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from ..kernels.linear import linear
+from .base import MATRIX, FeedForward, TensorSpec, place, register_part
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        self.dim = int(spec.options["dim"])
+        self.hidden_dim = int(spec.options["hidden_dim"])
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [
+            TensorSpec(self._name("gate_proj.weight"), (self.hidden_dim, self.dim)),
+            TensorSpec(self._name("up_proj.weight"), (self.hidden_dim, self.dim)),
+            TensorSpec(self._name("down_proj.weight"), (self.dim, self.hidden_dim)),
+        ]
+
+    def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
+        gate, up = tensors[self._name("gate_proj.weight")], tensors[self._name("up_proj.weight")]
+        self.w_gate_up = place(torch.cat([gate, up], dim=0), MATRIX, dtype, device)
+        self.w_down = place(tensors[self._name("down_proj.weight")], MATRIX, dtype, device)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return linear(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down)
+
+
+register_part("feed_forward", "swiglu", SwiGLU)

@@ -1,0 +1,76 @@
+"""Shared by the GPU tests: model folders from plain weights, trace running,
+and the tolerance rule."""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from plain_llama import plain_forward
+
+
+def save_model_folder(path: Path, config: Mapping, weights: Mapping[str, torch.Tensor],
+                      dtype: torch.dtype = torch.float32) -> Path:
+    from safetensors.torch import save_file
+
+    path.mkdir(parents=True, exist_ok=True)
+    with open(path / "config.json", "w") as f:
+        json.dump(dict(config), f)
+    save_file({k: v.to(dtype).contiguous() for k, v in weights.items()}, str(path / "model.safetensors"))
+    return path
+
+
+def make_runner(folder: Path, dtype: torch.dtype, page_size: int, max_tokens: int, max_requests: int = 4):
+    from fastgen_amd.engine import Model, ModelRunner
+
+    model = Model.from_folder(folder, dtype, "cuda:0")
+    return ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_requests)
+
+
+def run_trace(runner, trace, tokens: Mapping[str, List[int]]) -> Dict[str, torch.Tensor]:
+    """Logits of every fed token, per request ``[len, vocab]`` (fp32, CPU)."""
+    from fastgen_amd.engine import StepEntry
+
+    rows: Dict[str, List[torch.Tensor]] = {rid: [] for rid in tokens}
+    for entries, ends in trace:
+        step = [StepEntry(rid, tokens[rid][s : s + n], list(range(n))) for rid, s, n in entries]
+        logits = runner.step(step).cpu()
+        at = 0
+        for rid, s, n in entries:
+            assert len(rows[rid]) == s, f"{rid}: trace feeds position {s} after {len(rows[rid])}"
+            rows[rid].extend(logits[at : at + n])
+            at += n
+        for rid in ends:
+            runner.release(rid)
+        runner.cache.check()
+    return {rid: torch.stack(r) for rid, r in rows.items() if r}
+
+
+def plain_logits(weights, config, tokens: Mapping[str, List[int]], dtype=torch.float32) -> Dict[str, torch.Tensor]:
+    return {rid: plain_forward(weights, config, t, dtype) for rid, t in tokens.items()}
+
+
+def assert_close(got: Mapping[str, torch.Tensor], want: Mapping[str, torch.Tensor], dtype: torch.dtype,
+                 noise: Optional[Mapping[str, torch.Tensor]] = None, what: str = "") -> None:
+    """float32: the engine and the plain implementation differ by rounding of
+    fp32 sums only: 2e-5 of the largest logit.  bfloat16: ``noise`` is the plain
+    implementation run in bfloat16; the engine may be off the fp32 result by
+    twice what that run is off, and no more."""
+    for rid, w in want.items():
+        g = got[rid]
+        assert g.shape == w.shape, f"{what} {rid}: shape {tuple(g.shape)} vs {tuple(w.shape)}"
+        assert torch.isfinite(g).all(), f"{what} {rid}: non-finite logits"
+        scale = float(w.abs().max())
+        err = (g - w).abs().amax(dim=-1)  # per position
+        if dtype == torch.float32:
+            tol = 2e-5 * scale
+        else:
+            tol = 2.0 * float((noise[rid] - w).abs().max()) + 1e-3 * scale
+        worst = int(err.argmax())
+        assert float(err.max()) <= tol, (
+            f"{what} request {rid}: first position over tolerance is "
+            f"{int((err > tol).nonzero()[0])} of {len(err)}, worst {worst}: {float(err.max()):.3e} > {tol:.3e}"
+        )

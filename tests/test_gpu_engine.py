@@ -1,0 +1,184 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16,
+under every way of cutting the same requests into steps."""
+
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+from helpers import assert_close, make_runner, plain_logits, run_trace, save_model_folder
+from plain_llama import TINY_A, TINY_B, TINY_C, plain_forward, plain_random_weights
+
+pytestmark = pytest.mark.gpu
+
+REPO = Path(__file__).resolve().parent.parent
+DTYPES = [torch.float32, torch.bfloat16]
+# config, weight seed, page size, request lengths
+CASES = {
+    "A": (TINY_A, 0, 16, {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 1}),
+    "B": (TINY_B, 1, 32, {"a": 1, "b": 12, "c": 40, "d": 90, "e": 150, "f": 129}),
+    "C": (TINY_C, 2, 64, {"a": 70, "b": 200, "c": 2, "d": 64, "e": 131}),
+}
+
+
+def sharpen(weights, factor=10.0):
+    """Random N(0, 0.02) projections give nearly flat attention, which would
+    hide a key that is missed or read from a wrong page; larger q/k
+    projections make single scores stand out."""
+    return {k: v * factor if ("q_proj" in k or "k_proj" in k) else v for k, v in weights.items()}
+
+
+@pytest.fixture(scope="module", params=sorted(CASES))
+def case(request, tmp_path_factory):
+    cfg, seed, page, lengths = CASES[request.param]
+    weights = sharpen(plain_random_weights(cfg, seed))
+    # the bfloat16 engine sees bfloat16 weights; the plain runs get the same values
+    weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    folder = save_model_folder(tmp_path_factory.mktemp(f"tiny{request.param}"), cfg, weights)
+    g = torch.Generator().manual_seed(100 + seed)
+    tokens = {rid: torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for rid, n in lengths.items()}
+    want = plain_logits(weights, cfg, tokens)
+    noise = plain_logits(weights, cfg, tokens, torch.bfloat16)
+    return dict(cfg=cfg, page=page, lengths=lengths, folder=folder, tokens=tokens, want=want, noise=noise,
+                weights=weights)
+
+
+def _check(case, dtype, trace, max_tokens=None, what=""):
+    need = traces.max_live_tokens(trace, round_to=max(64, case["page"]))
+    runner = make_runner(case["folder"], dtype, case["page"], max_tokens or need)
+    got = run_trace(runner, trace, case["tokens"])
+    assert runner.cache.live_requests() == []
+    assert_close(got, case["want"], dtype, case["noise"], what)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole(case, dtype):
+    _check(case, dtype, traces.whole(case["lengths"]), what="whole")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_last_32_one_by_one(case, dtype):
+    _check(case, dtype, traces.tail(case["lengths"], 32), what="tail")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_portions_of_changing_size(case, dtype):
+    _check(case, dtype, traces.chunks(case["lengths"]), what="chunks")
+    _check(case, dtype, traces.chunks(case["lengths"], sizes=(2, 2, 3, 16, 1, 31, 33)), what="chunks2")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", [0, 1])
+def test_mixed_with_pages_used_again(case, dtype, seed):
+    trace = traces.mixed(case["lengths"], max_live=4, seed=seed)
+    assert any(len(e) >= 3 for e, _ in trace)
+    need = traces.max_live_tokens(trace, round_to=max(64, case["page"]))
+    total = sum(-(-n // 64) * 64 for n in case["lengths"].values())
+    assert need < total  # so few pages that finished requests' pages are used again
+    _check(case, dtype, trace, max_tokens=need, what=f"mixed{seed}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_token_by_token_from_the_first(case, dtype):
+    """The first tokens of a sequence, and long decoding: one token a step
+    from position 0 on."""
+    rid = max(case["lengths"], key=case["lengths"].get)
+    n = case["lengths"][rid]
+    trace = [([(rid, p, 1)], [rid] if p == n - 1 else []) for p in range(n)]
+    runner = make_runner(case["folder"], dtype, case["page"], 64 * -(-n // 64))
+    got = run_trace(runner, trace, case["tokens"])
+    assert_close(got, {rid: case["want"][rid]}, dtype, case["noise"], "one-by-one")
+
+
+def test_float32_does_not_depend_on_the_cut(case):
+    """In 32-bit the logits at a position are the same numbers however the
+    tokens were cut and batched (every reduction runs in an order fixed by
+    the row itself)."""
+    a = run_trace(make_runner(case["folder"], torch.float32, case["page"], 1024), traces.whole(case["lengths"]),
+                  case["tokens"])
+    b = run_trace(make_runner(case["folder"], torch.float32, case["page"], 1024),
+                  traces.mixed(case["lengths"], seed=3), case["tokens"])
+    for rid in a:
+        assert torch.equal(a[rid], b[rid]), rid
+
+
+def test_a_stale_or_foreign_page_is_never_read(case):
+    """Pages are poisoned with NaN before every step except where the live
+    requests hold tokens: what lies beyond a request's length, in free pages
+    or in other requests' pages, must not reach its logits."""
+    from fastgen_amd.engine import StepEntry
+
+    runner = make_runner(case["folder"], torch.float32, case["page"], 512)
+    for t in runner.storage.k + runner.storage.v:
+        t.fill_(float("nan"))
+    toks = case["tokens"]
+    rid = max(case["lengths"], key=case["lengths"].get)
+    n = case["lengths"][rid]
+    cut = n // 2
+    got = [runner.step([StepEntry(rid, toks[rid][:cut], list(range(cut)))])]
+    got.append(runner.step([StepEntry(rid, toks[rid][cut:], list(range(n - cut)))]))
+    got = torch.cat(got).cpu()
+    assert torch.isfinite(got).all()
+    assert_close({rid: got}, {rid: case["want"][rid]}, torch.float32, None, "poison")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_trace_run_program(case, dtype_name, tmp_path):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and
+    ``done`` lines out."""
+    dtype = getattr(torch, dtype_name)
+    trace = traces.mixed(case["lengths"], seed=5)
+    need = traces.max_live_tokens(trace, 64)
+    lines, wants = [], []
+    for i, (entries, ends) in enumerate(trace):
+        ents = []
+        for rid, s, n in entries:
+            want = list(range(n)) if i % 3 else ([n - 1] if n > 1 else [])  # sometimes only the last, or nothing
+            ents.append({"id": rid, "tokens": case["tokens"][rid][s : s + n], "want": want})
+            wants += [(i, rid, s + w) for w in want]
+        lines.append(json.dumps({"step": i, "entries": ents, "end": ends}))
+    out = tmp_path / "out"
+    cmd = [sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(case["folder"]), "--dtype", dtype_name,
+           "--out", str(out), "--max-tokens", str(need), "--page-size", str(case["page"])]
+    proc = subprocess.run(cmd, input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split() == [x for i in range(len(trace)) for x in ("done", str(i))]
+    V = case["cfg"]["vocab_size"]
+    got, want, noise = {}, {}, {}
+    by_step = {}
+    for i, rid, p in wants:
+        by_step.setdefault(i, []).append((rid, p))
+    for i, items in by_step.items():
+        arr = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, V)
+        assert arr.shape[0] == len(items)
+        for row, (rid, p) in zip(arr, items):
+            key = f"{rid}@{p}"
+            got[key] = torch.from_numpy(row.copy())[None]
+            want[key] = case["want"][rid][p][None]
+            noise[key] = case["noise"][rid][p][None]
+    for i in range(len(trace)):
+        assert (i in by_step) == (out / f"{i}.f32").exists()
+    assert_close(got, want, dtype, noise, "trace_run")
+
+
+def test_unsharpened_model_and_loader_round_trip(tmp_path):
+    """The random-weights mode writes a folder that the plain implementation
+    reads under checkpoint names; logits agree."""
+    from safetensors.torch import load_file
+
+    from fastgen_amd.weights import write_model_folder
+
+    folder = write_model_folder(tmp_path / "m", TINY_B, seed=11)
+    cfg = json.load(open(folder / "config.json"))
+    weights = load_file(str(folder / "model.safetensors"))
+    toks = {"x": list(range(3, 90))}
+    want = plain_logits(weights, cfg, toks)
+    runner = make_runner(folder, torch.float32, 16, 128)
+    got = run_trace(runner, traces.chunks({"x": 87}), toks)
+    assert_close(got, want, torch.float32, None, "written folder")

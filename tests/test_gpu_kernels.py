@@ -1,0 +1,346 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the
+engine tests' (head sizes in steps of 16, odd numbers of heads and groups,
+widths and vocabularies that are no power of two)."""
+
+import math
+
+import pytest
+import torch
+
+from plain_llama import (
+    plain_attention,
+    plain_rmsnorm,
+    plain_rope_frequencies,
+    plain_rope_interleaved,
+    plain_top_p_keep,
+)
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from fastgen_amd.kernels import ops as _ops
+
+    return _ops
+
+
+def tol(dtype):
+    return dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+# ------------------------------------------------------------------- rows
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,D,T", [(515, 240, 7), (1000, 4096, 3), (33, 24, 300)])
+def test_embed(ops, dtype, V, D, T):
+    torch.manual_seed(0)
+    table = torch.randn(V, D).to(dtype)
+    tok = torch.randint(0, V, (T,), dtype=torch.int32)
+    tok[0], tok[-1] = 0, V - 1
+    out = torch.empty(T, D, dtype=torch.float32, device=DEV)
+    ops.embed(table.to(DEV), tok.to(DEV), out)
+    assert torch.equal(out.cpu(), table[tok.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("T,D,eps", [(1, 4096, 1e-5), (5, 240, 3e-6), (300, 72, 1e-2), (3, 8200, 1e-6)])
+def test_add_rmsnorm(ops, dtype, wdtype, T, D, eps):
+    torch.manual_seed(1)
+    h = torch.randn(T, D) * 3
+    delta = torch.randn(T, D).to(dtype)
+    w = (1 + 0.1 * torch.randn(D)).to(wdtype)
+    hd, out = h.to(DEV), torch.empty(T, D, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(hd, delta.to(DEV), w.to(DEV), eps, out)
+    hsum = h + delta.float()
+    assert torch.equal(hd.cpu(), hsum)  # the residual sum is exact fp32
+    want = (hsum * torch.rsqrt((hsum * hsum).mean(-1, keepdim=True) + eps) * w.float()).to(dtype)
+    assert torch.allclose(out.cpu().float(), want.float(), **tol(dtype))
+    # without delta, and gathered rows (h untouched, a row may be named twice)
+    rows = torch.tensor([T - 1, 0, T - 1], dtype=torch.int32)
+    h2 = h.to(DEV)
+    out2 = torch.empty(3, D, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h2, delta.to(DEV), w.to(DEV), eps, out2, rows.to(DEV))
+    assert torch.equal(h2.cpu(), h)
+    assert torch.allclose(out2.cpu().float(), want[rows.long()].float(), **tol(dtype))
+    out3 = torch.empty(T, D, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h2, None, w.to(DEV), eps, out3)
+    assert torch.allclose(out3.cpu().float(), plain_rmsnorm(h, w.float(), eps).to(dtype).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_per_head_rows(ops, dtype):
+    torch.manual_seed(2)
+    x = torch.randn(6, 5, 48).to(dtype)  # a norm over head_dim, applied per head
+    w = torch.rand(48).to(dtype)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-6).cpu()
+    assert torch.allclose(got.float(), plain_rmsnorm(x, w, 1e-6).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,F", [(1, 14336), (9, 328), (70, 1000)])
+def test_silu_mul(ops, dtype, T, F):
+    torch.manual_seed(3)
+    gu = (torch.randn(T, 2 * F) * 4).to(dtype)
+    got = ops.silu_mul(gu.to(DEV)).cpu()
+    g, u = gu[:, :F].float(), gu[:, F:].float()
+    want = (g * torch.sigmoid(g) * u).to(dtype)
+    assert torch.allclose(got.float(), want.float(), **tol(dtype))
+
+
+# ------------------------------------------------------------- rope + write
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,rot,P", [(4, 2, 16, 16, 16), (5, 1, 48, 48, 32), (8, 8, 128, 128, 64),
+                                           (6, 3, 64, 32, 8), (3, 3, 80, 0, 16)])
+def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P):
+    torch.manual_seed(4)
+    T, n_pages = 37, 9
+    width = (H + 2 * KV) * hd
+    qkv = torch.randn(T, width).to(dtype)
+    pos = torch.randint(0, 5000, (T,), dtype=torch.int32)
+    freqs = plain_rope_frequencies(rot, 10000.0) if rot else None
+    slots = torch.randperm(n_pages * P)[:T].to(torch.int32)
+    slots[5] = -1  # a token whose k, v are not to be written
+    kp = torch.full((n_pages, KV, P, hd), 7.0, dtype=dtype)
+    vp = torch.full((n_pages, KV, hd, P), 7.0, dtype=dtype)
+    qkv_d, kp_d, vp_d = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    ops.rope_kv_write(qkv_d, pos.to(DEV), None if freqs is None else freqs.to(DEV), slots.to(DEV), kp_d, vp_d,
+                      H, KV, hd, rot)
+    q = qkv[:, : H * hd].view(T, H, hd)
+    k = qkv[:, H * hd : (H + KV) * hd].view(T, KV, hd)
+    v = qkv[:, (H + KV) * hd :].view(T, KV, hd)
+
+    def rotate(x):
+        if not rot:
+            return x
+        out = x.clone()
+        out[..., :rot] = plain_rope_interleaved(x[..., :rot], pos, freqs)
+        return out
+
+    got = qkv_d.cpu()
+    assert torch.allclose(got[:, : H * hd].float(), rotate(q).reshape(T, -1).float(), **tol(dtype))
+    assert torch.equal(got[:, (H + KV) * hd :], qkv[:, (H + KV) * hd :])  # v untouched in place
+    want_k, want_v = kp.clone(), vp.clone()
+    rk = rotate(k)
+    for t in range(T):
+        s = int(slots[t])
+        if s < 0:
+            continue
+        want_k[s // P, :, s % P, :] = rk[t]
+        want_v[s // P, :, :, s % P] = v[t]
+    assert torch.allclose(kp_d.cpu().float(), want_k.float(), **tol(dtype))
+    assert torch.equal(vp_d.cpu(), want_v)  # nothing else in the pool changed either
+
+
+# ---------------------------------------------------------------- attention
+def _paged_case(dtype, seqs, H, KV, hd, P, seed, poison=True, peak=None):
+    """``seqs``: list of (n_cached, n_new).  Returns device operands and the
+    per-sequence whole q, k, v on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(seqs)
+    pages_of = [-(-(a + b) // P) for a, b in seqs]
+    n_pages = sum(pages_of) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    fill = float("nan") if poison else 0.0
+    kp = torch.full((n_pages, KV, P, hd), fill, dtype=dtype)
+    vp = torch.full((n_pages, KV, hd, P), fill, dtype=dtype)
+    table = torch.zeros(B, max(pages_of), dtype=torch.int32)
+    qs, ks, vs, q_rows, seq_of, posv = [], [], [], [], [], []
+    for b, (n0, n1) in enumerate(seqs):
+        n = n0 + n1
+        q = torch.randn(n, H, hd, generator=g).to(dtype)
+        k = torch.randn(n, KV, hd, generator=g).to(dtype)
+        v = torch.randn(n, KV, hd, generator=g).to(dtype)
+        if peak is not None and b == peak[0]:
+            _, qpos, qh, kpos = peak  # one score made to stand out
+            k[kpos, qh // (H // KV)] = 0
+            k[kpos, qh // (H // KV), 0] = 12.0
+            q[qpos, qh] = 0
+            q[qpos, qh, 0] = 12.0 * math.sqrt(hd)
+        pages = [perm.pop() for _ in range(pages_of[b])]
+        table[b, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        for p in range(n):
+            kp[pages[p // P], :, p % P, :] = k[p]
+            vp[pages[p // P], :, :, p % P] = v[p]
+        qs.append(q), ks.append(k), vs.append(v)
+        q_rows.append(q[n0:].reshape(n1, H * hd))
+        seq_of += [b] * n1
+        posv += list(range(n0, n))
+    q_flat = torch.cat(q_rows)
+    dev = lambda t: t.to(DEV)
+    return dict(
+        q=dev(q_flat), kp=dev(kp), vp=dev(vp), table=dev(table),
+        seq_of=dev(torch.tensor(seq_of, dtype=torch.int32)), pos=dev(torch.tensor(posv, dtype=torch.int32)),
+        whole=(qs, ks, vs),
+    )
+
+
+def _plain_rows(case, seqs, window=None):
+    qs, ks, vs = case["whole"]
+    out = []
+    for (n0, n1), q, k, v in zip(seqs, qs, ks, vs):
+        o = plain_attention(q.float(), k.float(), v.float(), window)
+        out.append(o[n0:].reshape(n1, -1))
+    return torch.cat(out)
+
+
+ATT_SHAPES = [
+    # H, KV, hd, P
+    (4, 2, 16, 16),
+    (5, 1, 48, 32),
+    (6, 3, 32, 8),
+    (8, 2, 128, 64),
+    (3, 3, 80, 128),
+    (16, 2, 64, 16),
+    (2, 1, 256, 32),
+]
+ATT_SEQS = [(0, 1), (0, 70), (131, 1), (60, 9), (17, 2), (255, 1), (0, 129)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,hd,P", ATT_SHAPES)
+@pytest.mark.parametrize("window", [0, 37])
+def test_paged_attention_general(ops, dtype, H, KV, hd, P, window):
+    case = _paged_case(dtype, ATT_SEQS, H, KV, hd, P, seed=5)
+    out = torch.empty_like(case["q"])
+    ops.paged_attention_general(case["q"], out, case["kp"], case["vp"], case["table"], case["seq_of"],
+                                case["pos"], H, hd**-0.5, window)
+    want = _plain_rows(case, ATT_SEQS, window or None)
+    assert torch.isfinite(out).all()  # poison in unwritten slots never reaches the output
+    assert torch.allclose(out.cpu().float(), want, **(dict(atol=2e-5, rtol=1e-5) if dtype == torch.float32
+                                                       else dict(atol=1.5e-2, rtol=2e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_stands_out(ops, dtype):
+    """One key among hundreds, in an early page, gets nearly all the weight:
+    the output is that key's value, which a kernel that drops a page, a tile
+    or a tile's edge would miss."""
+    H, KV, hd, P = 4, 2, 64, 16
+    for kpos in (0, 15, 16, 63, 64, 300):
+        seqs = [(0, 3), (400, 1), (10, 2)]
+        case = _paged_case(dtype, seqs, H, KV, hd, P, seed=6, peak=(1, 400, 3, kpos))
+        out = torch.empty_like(case["q"])
+        ops.paged_attention_general(case["q"], out, case["kp"], case["vp"], case["table"], case["seq_of"],
+                                    case["pos"], H, hd**-0.5, 0)
+        v = case["whole"][2][1]
+        got = out.cpu().float()[3].view(H, hd)[3]
+        assert torch.allclose(got, v[kpos, 1].float(), atol=2e-2), kpos
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_window_edge(ops, dtype):
+    """The key just outside the window is made to stand out and must not be
+    seen; the key just inside must."""
+    H, KV, hd, P, w = 2, 1, 32, 16, 40
+    for kpos, seen in ((100 - w, False), (100 - w + 1, True)):
+        seqs = [(100, 1)]
+        case = _paged_case(dtype, seqs, H, KV, hd, P, seed=7, peak=(0, 100, 1, kpos))
+        out = torch.empty_like(case["q"])
+        ops.paged_attention_general(case["q"], out, case["kp"], case["vp"], case["table"], case["seq_of"],
+                                    case["pos"], H, hd**-0.5, w)
+        v = case["whole"][2][0]
+        got = out.cpu().float()[0].view(H, hd)[1]
+        assert torch.allclose(got, v[kpos, 0].float(), atol=2e-2) == seen
+        assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs, w), atol=2e-2)
+
+
+# --------------------------------------------------------------------- gemm
+@pytest.mark.parametrize("dtype,odtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 515, 240), (7, 64, 64), (65, 130, 17), (300, 33, 1000), (2, 4096, 328)])
+def test_gemm_nt(ops, dtype, odtype, M, N, K):
+    torch.manual_seed(8)
+    x, w = torch.randn(M, K).to(dtype), torch.randn(N, K).to(dtype)
+    got = ops.gemm_nt(x.to(DEV), w.to(DEV), out_dtype=odtype).cpu()
+    want = (x.double() @ w.double().T)
+    assert got.dtype == odtype
+    err = (got.double() - want).abs().max() / want.abs().max()
+    assert err < (2e-6 if odtype == torch.float32 else 1e-2)
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    torch.manual_seed(9)
+    x, w = torch.randn(70, 333), torch.randn(129, 333)
+    full = ops.gemm_nt(x.to(DEV), w.to(DEV)).cpu()
+    for rows in ([0], [69], list(range(3, 68))):
+        part = ops.gemm_nt(x[rows].to(DEV), w.to(DEV)).cpu()
+        assert torch.equal(part, full[rows])  # bit for bit
+
+
+# ----------------------------------------------------------------- sampling
+def test_argmax_lowest_index_wins(ops):
+    torch.manual_seed(10)
+    logits = torch.randn(5, 128256)
+    logits[0, 77] = logits[0, 100000] = 50.0
+    logits[1, -1] = 60.0
+    logits[2, 0] = 60.0
+    got = ops.sample(logits.to(DEV)).cpu()
+    assert got.tolist() == [77, 128255, 0, int(logits[3].argmax()), int(logits[4].argmax())]
+
+
+def test_sampling_follows_the_distribution(ops):
+    V, n = 37, 20000
+    torch.manual_seed(11)
+    row = torch.randn(V) * 2
+    temp = 0.8
+    logits = row[None].expand(n, V).contiguous().to(DEV)
+    t = torch.full((n,), temp, device=DEV)
+    seeds = torch.full((n,), 1234, dtype=torch.int64, device=DEV)
+    counters = torch.arange(n, dtype=torch.int64, device=DEV)
+    got = ops.sample(logits, t, None, seeds, counters).cpu()
+    probs = torch.softmax(row / temp, -1)
+    counts = torch.bincount(got.long(), minlength=V).float()
+    chi2 = ((counts - n * probs) ** 2 / (n * probs)).sum()
+    assert chi2 < 80, chi2  # 36 degrees of freedom: 80 is beyond the 99.99th percentile
+    # the same (seed, counter) gives the same token whatever else is in the batch
+    again = ops.sample(logits[100:103].contiguous(), t[:3], None, seeds[:3], counters[100:103].contiguous()).cpu()
+    assert torch.equal(again, got[100:103])
+    # temperature 0 rows are greedy inside a sampling batch
+    t2 = t.clone()
+    t2[:5] = 0
+    assert (ops.sample(logits, t2, None, seeds, counters).cpu()[:5] == int(row.argmax())).all()
+
+
+def test_top_p_keeps_the_reference_set(ops):
+    V, n = 515, 4000
+    torch.manual_seed(12)
+    row = torch.randn(V) * 3
+    for p in (0.3, 0.9):
+        probs = torch.softmax(row, -1)
+        keep = plain_top_p_keep(probs[None], p)[0]
+        logits = row[None].expand(n, V).contiguous().to(DEV)
+        got = ops.sample(logits, torch.ones(n, device=DEV), torch.full((n,), p, device=DEV),
+                         torch.full((n,), 7, dtype=torch.int64, device=DEV),
+                         torch.arange(n, dtype=torch.int64, device=DEV)).cpu().long()
+        assert keep[got].all()  # never a dropped token
+        seen = torch.zeros(V, dtype=torch.bool)
+        seen[got] = True
+        likely = keep & (probs * n > 20)
+        assert seen[likely].all()  # every kept token that should show up does
+
+
+def test_logprob(ops):
+    torch.manual_seed(13)
+    logits = torch.randn(4, 1000) * 5
+    tok = torch.tensor([0, 999, 5, 17], dtype=torch.int32)
+    got = ops.logprob(logits.to(DEV), tok.to(DEV)).cpu()
+    want = torch.log_softmax(logits, -1)[torch.arange(4), tok.long()]
+    assert torch.allclose(got, want, atol=1e-5)
+
+
+# ------------------------------------------------------------ refused sizes
+def test_kernels_refuse_what_they_cannot_take(ops):
+    from fastgen_amd.kernels import KernelArgumentError
+
+    q = torch.zeros(1, 2 * 20, device=DEV)
+    kp = torch.zeros(2, 1, 16, 20, device=DEV)
+    vp = torch.zeros(2, 1, 20, 16, device=DEV)
+    i = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelArgumentError, match="head size"):
+        ops.paged_attention_general(q, torch.empty_like(q), kp, vp, i.view(1, 1), i, i, 2, 1.0)
+    with pytest.raises(KernelArgumentError, match="GPU only"):
+        ops.silu_mul(torch.zeros(2, 4))
