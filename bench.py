@@ -1,0 +1,119 @@
+#!/usr/bin/python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
+heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
+llama3 rope scaling) with random bfloat16 weights.  A "step" is one decode
+step of a batch whose requests each hold a 2,048-token prompt; ``value`` is
+decoded tokens a second.  The same line carries the time of a 2,048-token
+prefill, the decode step's fraction of the HBM roofline, and decode at batch
+1 and 64.  Token ids are uniform random (synthetic); nothing is read from disk.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM = 8.0e12  # bytes/s, MI355X published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_8B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
+    num_attention_heads=32, num_key_value_heads=8, rms_norm_eps=1e-5, vocab_size=128256, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=False, max_position_embeddings=131072,
+)
+FULL_LAYERS = 32
+PROMPT_LEN = 2048
+CONTEXT_LEN = 8192  # capacity per request
+PAGE = 64
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported", flush=True)
+        return 2
+
+    import torch
+
+    from fastgen_amd.engine import Engine
+
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[a.dtype]
+    cfg = dict(LLAMA_8B, num_hidden_layers=a.layers)
+    batches = sorted({a.batch} | (set() if a.no_points else {1, 64}))
+    max_b = max(batches)
+    t0 = time.time()
+    engine = Engine.from_config(cfg, seed=2, dtype=dtype, page_size=PAGE,
+                                max_tokens=max_b * (PROMPT_LEN + 512), max_batch=max_b,
+                                max_step_tokens=PROMPT_LEN)
+    torch.cuda.synchronize()
+    print(f"[bench] model built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    model = engine.model
+    D, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    H, KV = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    hd, L = D // H, a.layers
+    esize = 2 if a.dtype == "bf16" else 4
+    layer_params = D * (H + 2 * KV) * hd + H * hd * D + 3 * D * F
+    kv_bytes_per_token = 2 * KV * hd * esize * L
+
+    g = torch.Generator().manual_seed(0)
+
+    def prompt(n):
+        return torch.randint(0, V, (n,), generator=g).tolist()
+
+    # ------------------------------------------------------------ prefill
+    pre = engine.time_prefill(prompt(PROMPT_LEN), repeats=3)
+    T = PROMPT_LEN
+    flops = 2 * T * L * layer_params + L * 4 * H * hd * (T * (T + 1) // 2) + 2 * D * V
+    prefill = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
+               "frac": round(flops / pre / PEAK_FLOPS[a.dtype], 4)}
+    print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+
+    # ------------------------------------------------------------- decode
+    results = {}
+    for b in batches:
+        steps, warm = (a.steps, a.warmup)
+        dt = engine.time_decode([prompt(PROMPT_LEN) for _ in range(b)], steps=steps, warmup=warm)
+        ctx = PROMPT_LEN + warm + steps / 2  # mean cached tokens during the timed steps
+        nbytes = (L * layer_params + D * V) * esize + b * ctx * kv_bytes_per_token
+        results[b] = dict(tok_s=b * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9)
+        print(f"[bench] decode batch {b}: {results[b]}", file=sys.stderr, flush=True)
+
+    r = results[a.batch]
+    line = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2048 tokens; % of roofline",
+        "value": round(r["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(r["ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": a.dtype, "data": "synthetic",
+        "config": {
+            "model": "llama-3.1-8b-shape-random", "global_batch": a.batch, "seq_len": CONTEXT_LEN,
+            "prompt_len": PROMPT_LEN, "parallelism": "none", "layers": L, "layers_full": FULL_LAYERS,
+            "hidden": D, "heads": H, "kv_heads": KV, "head_dim": hd, "ffn": F, "vocab": V, "page_size": PAGE,
+            "rope_theta": cfg["rope_theta"], "rope_factor": 8.0, "norm_eps": cfg["rms_norm_eps"],
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": round(r["gbs"] * 1e9 / PEAK_HBM, 4)},
+        "points": {f"decode_b{b}": round(v["tok_s"], 1) for b, v in results.items() if b != a.batch},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

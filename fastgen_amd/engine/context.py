@@ -51,6 +51,7 @@ class StepContext:
     # host copies, for decisions about grids and kernels
     q_lens: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     n_cached: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
+    slot_ids_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     n_out: int = 0
 
     @property
@@ -110,5 +111,5 @@ def build_context(entries: Sequence[StepEntry], cache: CacheManager, act_dtype: 
     return StepContext(
         n_tokens=T, n_seqs=B, act_dtype=act_dtype, tokens=part[0], positions=part[1], seq_of_token=part[2],
         q_start=part[3], kv_len=part[4], slot_ids=part[5], out_rows=part[6], groups=groups, q_lens=q_lens,
-        n_cached=n_cached, n_out=len(out_rows),
+        n_cached=n_cached, slot_ids_host=slot_ids, n_out=len(out_rows),
     )

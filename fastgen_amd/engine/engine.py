@@ -1,0 +1,151 @@
+"""The engine: a model with its cache, the scheduler above the step function,
+and sampling.  ``add_request`` / ``step`` for a serving loop, ``generate`` for
+a batch of prompts.  (The reference's counterpart is ``Fastgen`` in
+``fastgen/generate.py:138-475``; ``fastgen_amd.generate`` offers that
+interface on top of this class.)
+"""
+
+from __future__ import annotations
+
+import time
+from pathlib import Path
+from typing import Any, Dict, Hashable, Iterable, List, Mapping, Optional, Sequence
+
+import torch
+
+from ..sampling import Sampler, SamplingParams
+from .context import StepEntry
+from .model import Model
+from .runner import ModelRunner
+from .scheduler import PlannedEntry, Request, Scheduler
+
+
+class Engine:
+    def __init__(self, model: Model, page_size: int = 64, max_tokens: int = 8192, max_batch: int = 64,
+                 max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0) -> None:
+        self.model = model
+        self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch)
+        cap = getattr(model.args, "max_position", 0) or None
+        if max_seq is None:
+            max_seq = cap
+        elif cap:
+            max_seq = min(max_seq, cap)
+        self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit)
+        self.sampler = Sampler(model.device)
+        self.seed = seed
+        self._n_requests = 0
+        self.n_steps = 0
+
+    # -------------------------------------------------------------- build
+    @classmethod
+    def from_folder(cls, model_dir: str | Path, dtype: torch.dtype = torch.bfloat16, device: str = "cuda:0",
+                    **kw: Any) -> "Engine":
+        return cls(Model.from_folder(model_dir, dtype, device), **kw)
+
+    @classmethod
+    def from_config(cls, config: Mapping[str, Any], seed: int, dtype: torch.dtype = torch.bfloat16,
+                    device: str = "cuda:0", **kw: Any) -> "Engine":
+        """A model of this configuration with seeded random weights."""
+        return cls(Model.random(config, seed, dtype, device), **kw)
+
+    # ------------------------------------------------------------ serving
+    def add_request(self, prompt: Sequence[int], params: SamplingParams = SamplingParams(),
+                    rid: Optional[Hashable] = None) -> Hashable:
+        rid = self._n_requests if rid is None else rid
+        vocab = self.model.vocab_size
+        if any(not 0 <= int(t) < vocab for t in prompt):
+            raise ValueError(f"request {rid!r}: token id outside [0, {vocab})")
+        # a request's own seed, unless it gave one: the engine's seed and its arrival number
+        seed = params.seed if params.seed else (self.seed * 1000003 + self._n_requests + 1)
+        self._n_requests += 1
+        self.scheduler.add(Request(
+            rid=rid, prompt=[int(t) for t in prompt], max_new=params.max_new_tokens,
+            temperature=float(params.temperature), top_p=float(params.top_p), seed=seed,
+            stop_ids=tuple(params.stop_ids), want_logprobs=params.logprobs,
+        ))
+        return rid
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def step(self) -> List[Request]:
+        """One step of the model over what the scheduler picks; the requests
+        that ended with it."""
+        plan = self.scheduler.plan()
+        done: List[Request] = []
+        if plan:
+            entries, rows = [], []
+            for e in plan:
+                toks = e.request.all_tokens()[e.start : e.start + e.n]
+                entries.append(StepEntry(e.request.rid, toks, [e.n - 1] if e.wants_logits else []))
+                if e.wants_logits:
+                    rows.append(e.request)
+            logits = self.runner.step(entries)
+            sampled: List[int] = []
+            lps = None
+            if rows:
+                tok = self.sampler.sample(
+                    logits, [r.temperature for r in rows], [r.top_p for r in rows], [r.seed for r in rows],
+                    [len(r.generated) for r in rows],
+                )
+                if any(r.want_logprobs for r in rows):
+                    lps = self.sampler.logprobs(logits, tok).tolist()
+                sampled = tok.tolist()
+            done = self.scheduler.commit(plan, sampled, lps)
+            self.n_steps += 1
+        # requests the scheduler ended while planning (alone and out of pages)
+        for r in self.scheduler.finished:
+            if r not in done:
+                done.append(r)
+        self.scheduler.finished.clear()
+        return done
+
+    def generate(self, prompts: Sequence[Sequence[int]], params: SamplingParams | Sequence[SamplingParams] = SamplingParams(),
+                 ) -> List[List[int]]:
+        """Generated ids for every prompt, in the order of the prompts."""
+        plist = list(params) if isinstance(params, (list, tuple)) else [params] * len(prompts)
+        rids = [self.add_request(p, sp) for p, sp in zip(prompts, plist)]
+        out: Dict[Hashable, List[int]] = {}
+        while self.has_work():
+            for r in self.step():
+                out[r.rid] = r.generated
+        return [out[r] for r in rids]
+
+    # ------------------------------------------------------- measurement
+    def time_prefill(self, prompt: Sequence[int], repeats: int = 3) -> float:
+        """Seconds of one step that takes the whole prompt and returns the
+        logits of its last token (best of ``repeats`` after one warm-up)."""
+        best = float("inf")
+        for i in range(repeats + 1):
+            rid = ("prefill-timing", i)
+            entry = StepEntry(rid, list(prompt), [len(prompt) - 1])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            self.runner.step([entry])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            self.runner.release(rid)
+            if i:
+                best = min(best, dt)
+        return best
+
+    def time_decode(self, prompts: Sequence[Sequence[int]], steps: int, warmup: int) -> float:
+        """Seconds of exactly ``steps`` decode steps of the batch ``prompts``
+        (greedy, no stop ids), after the prompts are in the cache and after
+        ``warmup`` untimed decode steps."""
+        params = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 1)
+        for p in prompts:
+            self.add_request(p, params)
+        while any(r.remaining() > 1 for r in self.scheduler.running) or self.scheduler.waiting:
+            self.step()
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        while self.has_work():
+            self.step()
+        return dt

@@ -1,0 +1,215 @@
+"""The scheduler: which requests run in the next step, and with how many
+tokens each.  Host-only; it talks to the cache manager and to nothing on a
+device, so its decisions can be tested without a GPU.
+
+Policy, after ``fastgen/generate.py:477-613`` with one change: the reference
+runs a decode round and then a separate prefill phase cut every
+``max_prefill`` tokens (``801-851``); here every step has one token budget,
+spent first on one token for each decoding request and then on prompt
+portions in arrival order, so prompt portions ride beside decoded tokens.
+
+* Admission is first come, first served, preempted requests before new ones
+  (``540-572``), while fewer than ``max_batch`` requests are live and the
+  free pages hold the request's known tokens plus one.
+* When a decoding request needs a page and none is free, the request admitted
+  last is preempted: its pages go back, it returns to the head of the waiting
+  line and is later recomputed from its prompt and everything it generated
+  (``497-502``, ``772``).  A request that is alone and still out of pages ends
+  there with reason ``"cache_full"`` (the reference lets it run into its
+  length cap, ``509-513``).
+* A request ends when it samples a stop id, has ``max_new`` tokens, or reaches
+  ``max_seq`` tokens (``95-113``, ``445-447``, ``637-662``).
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
+
+from ..cache.manager import CacheManager
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    max_new: int
+    temperature: float = 0.0
+    top_p: float = 1.0
+    seed: int = 0
+    stop_ids: Tuple[int, ...] = ()
+    want_logprobs: bool = False
+    generated: List[int] = field(default_factory=list)
+    logprobs: List[float] = field(default_factory=list)
+    n_fed: int = 0  # tokens of prompt + generated whose keys are in the cache
+    preemptions: int = 0
+    finish_reason: Optional[str] = None
+
+    def all_tokens(self) -> List[int]:
+        return self.prompt + self.generated
+
+    def n_known(self) -> int:
+        return len(self.prompt) + len(self.generated)
+
+    def remaining(self) -> int:
+        """Known tokens not yet in the cache; feeding the last one yields the
+        logits of the next token."""
+        return self.n_known() - self.n_fed
+
+
+@dataclass
+class PlannedEntry:
+    request: Request
+    start: int  # index into all_tokens()
+    n: int
+    wants_logits: bool  # this portion ends at the last known token
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_batch: int, max_step_tokens: int,
+                 max_seq: Optional[int] = None, on_admit: Optional[Callable[[Hashable], None]] = None) -> None:
+        if max_batch < 1 or max_step_tokens < 1:
+            raise ValueError("max_batch and max_step_tokens must be at least 1")
+        self.cache = cache
+        self.max_batch = min(max_batch, cache.n_slots)
+        self.max_step_tokens = max_step_tokens
+        pool_tokens = min(cache.n_pages) * cache.page_size if cache.n_groups else 1 << 62
+        self.max_seq = min(max_seq or pool_tokens, pool_tokens)
+        self._admit = on_admit or cache.admit
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []  # in order of admission
+        self.finished: List[Request] = []
+        self.n_preemptions = 0
+
+    # ------------------------------------------------------------- intake
+    def add(self, req: Request) -> None:
+        if not req.prompt:
+            raise ValueError(f"request {req.rid!r}: empty prompt")
+        if len(req.prompt) + 1 > self.max_seq:
+            raise ValueError(
+                f"request {req.rid!r}: a prompt of {len(req.prompt)} tokens can never fit"
+                f" (at most {self.max_seq} tokens a request)"
+            )
+        if req.max_new < 1:
+            raise ValueError(f"request {req.rid!r}: max_new must be at least 1")
+        self.waiting.append(req)
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # --------------------------------------------------------------- plan
+    def _preempt(self, victim: Request) -> None:
+        self.cache.release(victim.rid)
+        victim.n_fed = 0
+        victim.preemptions += 1
+        self.n_preemptions += 1
+        self.running.remove(victim)
+        self.waiting.appendleft(victim)
+
+    def _finish(self, req: Request, reason: str) -> None:
+        req.finish_reason = reason
+        if self.cache.is_live(req.rid):
+            self.cache.release(req.rid)
+        if req in self.running:
+            self.running.remove(req)
+        self.finished.append(req)
+
+    def _fits(self, req: Request, n: int) -> int:
+        """The largest ``m <= n`` such that ``m`` more tokens of ``req`` fit in
+        the pages it holds plus the free ones."""
+        lo = 0
+        for g in range(self.cache.n_groups):
+            held = self.cache.n_table_entries(req.rid, g)
+            room = (held + self.cache.free_pages(g)) * self.cache.page_size - self.cache.length(req.rid)
+            n = min(n, room)
+        return max(lo, n)
+
+    def plan(self) -> List[PlannedEntry]:
+        entries: List[PlannedEntry] = []
+        budget = self.max_step_tokens
+        # A. one token for every decoding request, oldest first; make room by
+        #    preempting the youngest
+        for req in list(self.running):
+            if budget == 0:
+                break
+            if req not in self.running or req.remaining() != 1:
+                continue
+            while not self.cache.can_reserve(req.rid, 1):
+                victim = self.running[-1]
+                if victim is req and len(self.running) == 1:
+                    self._finish(req, "cache_full")
+                    break
+                # an entry already planned for the victim is withdrawn
+                entries = [e for e in entries if e.request is not victim]
+                self._preempt(victim)
+                if victim is req:
+                    break
+            if req not in self.running:
+                continue
+            self.cache.reserve(req.rid, 1)
+            entries.append(PlannedEntry(req, req.n_fed, 1, True))
+            budget -= 1
+        budget = self.max_step_tokens - sum(e.n for e in entries)
+        # B. portions of prompts already admitted, oldest first
+        for req in self.running:
+            if budget == 0:
+                break
+            rem = req.remaining()
+            if rem < 1 or any(e.request is req for e in entries):
+                continue
+            n = self._fits(req, min(rem, budget))
+            if n < 1:
+                continue
+            self.cache.reserve(req.rid, n)
+            entries.append(PlannedEntry(req, req.n_fed, n, n == rem))
+            budget -= n
+        # C. admission: preempted requests first (they sit at the head), then new ones
+        while self.waiting and len(self.running) < self.max_batch and budget > 0:
+            req = self.waiting[0]
+            need = req.n_known() + 1
+            if any(self.cache.pages_needed_fresh(need, g) > self.cache.free_pages(g)
+                   for g in range(self.cache.n_groups)):
+                break
+            self.waiting.popleft()
+            self._admit(req.rid)
+            self.running.append(req)
+            n = min(req.remaining(), budget)
+            self.cache.reserve(req.rid, n)
+            entries.append(PlannedEntry(req, req.n_fed, n, n == req.remaining()))
+            budget -= n
+        # D. nothing can move although requests are live: the pages are all
+        #    held by half-fed prompts; the youngest gives way
+        if not entries and len(self.running) > 1:
+            self._preempt(self.running[-1])
+            return self.plan()
+        return entries
+
+    # ------------------------------------------------------------- commit
+    def commit(self, entries: Sequence[PlannedEntry], sampled: Sequence[int],
+               logprobs: Optional[Sequence[float]] = None) -> List[Request]:
+        """Record what the step did: ``sampled`` holds one token for every
+        entry that wanted logits, in order.  Returns the requests that ended."""
+        done: List[Request] = []
+        it = iter(range(len(sampled)))
+        for e in entries:
+            req = e.request
+            req.n_fed += e.n
+            if not e.wants_logits:
+                continue
+            i = next(it)
+            tok = int(sampled[i])
+            req.generated.append(tok)
+            if logprobs is not None and req.want_logprobs:
+                req.logprobs.append(float(logprobs[i]))
+            if tok in req.stop_ids:
+                reason = "stop"
+            elif len(req.generated) >= req.max_new:
+                reason = "length"
+            elif req.n_known() >= self.max_seq:
+                reason = "max_seq"
+            else:
+                continue
+            self._finish(req, reason)
+            done.append(req)
+        return done

@@ -1,0 +1,139 @@
+"""The reference's programming interface on top of the engine:
+``GenArgs``, ``Packet`` and ``Fastgen.build(...).generate(queue)``
+(``fastgen/generate.py:30-76, 138-173, 405-475``), with the same names and
+meanings of options where the reference has them.
+
+    fg = Fastgen.build(model_dir, GenArgs(max_batch=8, max_gen=64))
+    q = queue.Queue(); q.put(Packet(thread_id=0, tokens=[1, 2, 3])); q.put(None)
+    for pkt in fg.generate(q):
+        print(pkt.thread_id, pkt.tokens)
+"""
+
+from __future__ import annotations
+
+import logging
+import queue
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Any, Iterator, List, Optional, Sequence
+
+import torch
+
+from .engine import Engine, Model
+from .sampling import SamplingParams
+
+logger = logging.getLogger(__name__)
+
+
+@dataclass
+class GenArgs:
+    """Generation options (``fastgen/generate.py:30-59``).  Options of the
+    reference that belong to parts this engine does not have (host cache,
+    CUDA graphs count, fp8, hold-back thresholds) are absent."""
+
+    use_sampling: bool = True  # else greedy for every request
+    temperature: float = 0.7
+    top_p: float = 0.9
+    logprobs: bool = False
+    max_batch: int = 256  # most concurrent requests
+    max_seq: int = -1  # cache size in tokens, also the cap of one request; negative: from gpu_gb
+    max_gen: Optional[int] = None  # default cap of generated tokens
+    cache_block: int = 64  # tokens per cache page (the reference's default is 256)
+    max_prefill: int = 8192  # token budget of one step
+    prefill_gb: float = 0.5  # activation budget, used when sizing the cache
+    gpu_gb: float = 20  # memory budget, used when max_seq is negative
+    seed: int = 777  # the reference's tools seed the global generator with 777 (tools/chat.py:47)
+    dtype: torch.dtype = torch.bfloat16
+
+
+@dataclass
+class Packet:
+    """A request going in, a generation coming out (``fastgen/generate.py:62-76``)."""
+
+    thread_id: Any
+    tokens: List[int] = field(default_factory=list)
+    temperature: Optional[float] = None
+    logprobs: Optional[List[float]] = None
+    max_gen: Optional[int] = None
+
+
+def cache_tokens_for_budget(model: Model, gen_args: GenArgs, bytes_per_token: int) -> int:
+    """``fastgen/utils/tune.py:68-84``: what is left of ``gpu_gb`` after the
+    weights and the activation budget, in tokens of cache, rounded up to a page."""
+    left = gen_args.gpu_gb * 1e9 - model.weight_bytes() - gen_args.prefill_gb * 1e9
+    tokens = int(left // max(1, bytes_per_token))
+    if tokens < gen_args.cache_block:
+        raise RuntimeError(
+            f"gpu_gb={gen_args.gpu_gb} leaves no room for one cache page beside"
+            f" {model.weight_bytes() / 1e9:.2f} GB of weights"
+        )
+    return -(-tokens // gen_args.cache_block) * gen_args.cache_block
+
+
+class Fastgen:
+    def __init__(self, engine: Engine, gen_args: GenArgs, stop_tokens: Sequence[int] = ()) -> None:
+        self.engine, self.gen_args, self.stop_tokens = engine, gen_args, tuple(stop_tokens)
+
+    @classmethod
+    def build(cls, model_dir: str | Path, gen_args: GenArgs = GenArgs(), device: str = "cuda:0",
+              stop_tokens: Optional[Sequence[int]] = None) -> "Fastgen":
+        """Load the model of ``model_dir`` and size its cache
+        (``fastgen/generate.py:139-173``)."""
+        device_ = torch.device(device)
+        if device_.type != "cuda":
+            raise RuntimeError("fastgen_amd runs on a GPU only")  # generate.py:148
+        model = Model.from_folder(model_dir, gen_args.dtype, device_)
+        if stop_tokens is None:
+            eos = getattr(model.args, "extra", {}).get("eos_token_id", [])
+            stop_tokens = eos if isinstance(eos, (list, tuple)) else [eos]
+        max_seq = gen_args.max_seq
+        if max_seq < 0:
+            esize = torch.empty((), dtype=gen_args.dtype).element_size()
+            per_token = sum(2 * n.n_kv_heads * n.head_dim * esize for n in model.paged_needs() if n is not None)
+            max_seq = cache_tokens_for_budget(model, gen_args, per_token)
+        max_batch = max(1, min(gen_args.max_batch, max_seq // gen_args.cache_block))  # generate.py:234-236
+        logger.info("cache of %d tokens in pages of %d, at most %d requests", max_seq, gen_args.cache_block, max_batch)
+        engine = Engine(model, page_size=gen_args.cache_block, max_tokens=max_seq, max_batch=max_batch,
+                        max_step_tokens=gen_args.max_prefill, max_seq=max_seq, seed=gen_args.seed)
+        return cls(engine, gen_args, stop_tokens)
+
+    def _params(self, pkt: Packet) -> SamplingParams:
+        ga = self.gen_args
+        # as in the reference a packet's temperature of None or 0 falls back to
+        # the default (generate.py:790); greedy is the global switch (892)
+        temp = (pkt.temperature or ga.temperature) if ga.use_sampling else 0.0
+        max_gen = pkt.max_gen or ga.max_gen or (self.engine.scheduler.max_seq - len(pkt.tokens))
+        return SamplingParams(temperature=temp, top_p=ga.top_p, max_new_tokens=max(1, max_gen),
+                              stop_ids=self.stop_tokens, logprobs=ga.logprobs)
+
+    def generate(self, q: "queue.Queue[Optional[Packet]]") -> Iterator[Packet]:
+        """Packets from ``q`` in, finished packets out, in the order they
+        finish; ``None`` on the queue ends the input, and what is in flight
+        completes (``fastgen/generate.py:405-425``).  Blocks on the queue only
+        when nothing is in flight (547)."""
+        eoq = False
+        pending = {}
+        while True:
+            while not eoq:
+                try:
+                    pkt = q.get(block=not self.engine.has_work())
+                except queue.Empty:
+                    break
+                if pkt is None:
+                    eoq = True
+                    break
+                rid = self.engine.add_request(pkt.tokens, self._params(pkt))
+                pending[rid] = pkt
+            if not self.engine.has_work():
+                if eoq:
+                    return
+                continue
+            for req in self.engine.step():
+                src = pending.pop(req.rid)
+                yield Packet(thread_id=src.thread_id, tokens=list(req.generated), temperature=src.temperature,
+                             logprobs=list(req.logprobs) if self.gen_args.logprobs else None, max_gen=src.max_gen)
+
+    def destroy(self) -> None:
+        """Give the GPU memory back (``fastgen/generate.py:355-362``)."""
+        self.engine = None  # type: ignore[assignment]
+        torch.cuda.empty_cache()

@@ -1,0 +1,52 @@
+"""Choice of the next token from fp32 logits.
+
+The reference (``fastgen/generate.py:887-896``, ``utils/sampling.py:6-31``):
+greedy is ``argmax``; otherwise ``softmax(logits / temperature)`` and either a
+plain multinomial draw (``top_p >= 1``) or a draw from the nucleus.  One global
+switch decides greedy or not, and one global generator feeds every request.
+Here every request carries its own temperature (0 = greedy), nucleus and seed;
+the uniform number for its ``k``-th generated token is a function of
+``(seed, k)`` alone, so what a request samples does not depend on its
+batch-mates or on how its prompt was cut.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from ..kernels import ops
+
+
+@dataclass(frozen=True)
+class SamplingParams:
+    temperature: float = 0.0
+    top_p: float = 1.0
+    seed: int = 0
+    max_new_tokens: int = 16
+    stop_ids: Tuple[int, ...] = ()
+    logprobs: bool = False
+
+
+class Sampler:
+    """Batches the per-request parameters and calls the sampling kernel."""
+
+    def __init__(self, device: torch.device | str) -> None:
+        self.device = torch.device(device)
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
+               seeds: Sequence[int], counters: Sequence[int]) -> torch.Tensor:
+        """int32 ``[n]`` on the device; row ``i`` is greedy if ``temperatures[i] == 0``."""
+        n = logits.shape[0]
+        if not any(t > 0 for t in temperatures):
+            return ops.sample(logits)
+        packed_f = torch.tensor([list(temperatures), list(top_ps)], dtype=torch.float32).to(self.device)
+        mask = (1 << 63) - 1
+        packed_i = torch.tensor([[s & mask for s in seeds], list(counters)], dtype=torch.int64).to(self.device)
+        top_p = packed_f[1] if any(p < 1.0 for p in top_ps) else None
+        return ops.sample(logits, packed_f[0], top_p, packed_i[0], packed_i[1])
+
+    def logprobs(self, logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+        return ops.logprob(logits, tokens)

@@ -1,0 +1,112 @@
+"""``fgchat``: the reference's command line (``fastgen/tools/chat.py:87-216``)
+with its option names, generating in-process.  Without a prompt option it is
+the reference's dialogue loop (needs a tokenizer in the model folder; ``/q``
+quits, ``/r`` drops the last exchange); with one it generates once and exits:
+
+    fgchat MODEL --prompt-ids 1,2,3 --max-tokens 32 --temperature 0
+    fgchat MODEL --random-prompt 128 --max-tokens 64
+"""
+
+from __future__ import annotations
+
+import argparse
+import logging
+import queue
+import sys
+import time
+from typing import List, Optional
+
+import torch
+
+
+def build_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="fgchat", description="Generate with a model folder on one MI355X.")
+    ap.add_argument("model", help="model folder (config.json, safetensors, optionally tokenizer.json)")
+    ap.add_argument("--temperature", type=float, default=0.7, help="0 is greedy (default 0.7)")
+    ap.add_argument("--top-p", type=float, default=1.0)
+    ap.add_argument("--max-tokens", type=int, default=None, help="most tokens to generate")
+    ap.add_argument("--gpu-gb", type=float, default=20, help="memory budget for weights and cache")
+    ap.add_argument("--tensor-parallel", type=int, default=1, help="accepted for compatibility; must be 1")
+    ap.add_argument("--verbose", action="store_true")
+    # beyond the reference: generate once without a dialogue
+    ap.add_argument("--prompt", help="text prompt (needs tokenizer.json in the model folder)")
+    ap.add_argument("--prompt-ids", help="comma-separated token ids")
+    ap.add_argument("--random-prompt", type=int, metavar="LEN", help="a prompt of LEN uniform random ids")
+    ap.add_argument("--seed", type=int, default=777)
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--page-size", type=int, default=64)
+    ap.add_argument("--max-seq", type=int, default=-1, help="cache size in tokens (default: from --gpu-gb)")
+    ap.add_argument("--max-step-tokens", type=int, default=8192, help="token budget of one step")
+    return ap
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    from ..generate import Fastgen, GenArgs, Packet
+    from .tokenizer import FolderTokenizer
+
+    a = build_parser().parse_args(argv)
+    if a.tensor_parallel != 1:
+        print("fgchat: this engine runs on one GPU; --tensor-parallel must be 1", file=sys.stderr)
+        return 2
+    logging.basicConfig(level=logging.INFO if a.verbose else logging.WARNING)
+    tokenizer = FolderTokenizer.maybe(a.model)
+    gen_args = GenArgs(
+        use_sampling=bool(a.temperature), temperature=a.temperature, top_p=a.top_p, max_batch=1,
+        max_gen=a.max_tokens, gpu_gb=a.gpu_gb, cache_block=a.page_size, max_seq=a.max_seq,
+        max_prefill=a.max_step_tokens, seed=a.seed, dtype=getattr(torch, a.dtype),
+    )
+    fg = Fastgen.build(a.model, gen_args, stop_tokens=tokenizer.stop_tokens if tokenizer else None)
+    q: "queue.Queue" = queue.Queue()
+    gen = fg.generate(q)
+
+    def run(tokens: List[int]) -> List[int]:
+        t0 = time.time()
+        q.put(Packet(thread_id=0, tokens=tokens))
+        pkt = next(gen)
+        dt = time.time() - t0
+        print(f"[{len(pkt.tokens)} tokens, {len(pkt.tokens) / dt:.1f} tok/s]", file=sys.stderr)
+        return pkt.tokens
+
+    one_shot = a.prompt is not None or a.prompt_ids is not None or a.random_prompt is not None
+    if one_shot:
+        if a.prompt is not None:
+            if tokenizer is None:
+                print("fgchat: --prompt needs tokenizer.json in the model folder", file=sys.stderr)
+                return 2
+            ids = tokenizer.encode_dialog([{"role": "user", "content": a.prompt}])
+        elif a.prompt_ids is not None:
+            ids = [int(x) for x in a.prompt_ids.replace(" ", "").split(",") if x]
+        else:
+            g = torch.Generator().manual_seed(a.seed)
+            ids = torch.randint(0, fg.engine.model.vocab_size, (a.random_prompt,), generator=g).tolist()
+        out = run(ids)
+        print(",".join(str(t) for t in out))
+        if tokenizer is not None:
+            print(tokenizer.decode([t for t in out if t not in tokenizer.stop_tokens]))
+        return 0
+    if tokenizer is None:
+        print("fgchat: a dialogue needs tokenizer.json in the model folder; use --prompt-ids or --random-prompt",
+              file=sys.stderr)
+        return 2
+    dialog: List[dict] = []
+    while True:
+        try:
+            line = input("> ")
+        except EOFError:
+            return 0
+        if line.strip() == "/q":
+            return 0
+        if line.strip() == "/r":
+            dialog = dialog[:-2]
+            continue
+        dialog.append({"role": "user", "content": line})
+        out = run(tokenizer.encode_dialog(dialog))
+        if out and out[-1] in tokenizer.stop_tokens:
+            out = out[:-1]  # tools/chat.py:205-206
+        text = tokenizer.decode(out)
+        print(text)
+        dialog.append({"role": "assistant", "content": text})
+
+
+if __name__ == "__main__":
+    sys.exit(main())

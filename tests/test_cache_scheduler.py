@@ -1,0 +1,267 @@
+"""The cache manager's bookkeeping and the scheduler's decisions (no GPU).
+The scheduler is driven with a stand-in for the model that "samples" a fixed
+function of the request and position, so its plans can be checked exactly."""
+
+import random
+
+import pytest
+
+from fastgen_amd.cache import RELEASED, CacheManager, OutOfPages, OutOfSlots
+from fastgen_amd.engine.scheduler import Request, Scheduler
+
+
+# ------------------------------------------------------------ cache manager
+def test_pages_follow_the_length():
+    c = CacheManager(16, [8], [None], n_slots=2)
+    c.admit("a")
+    c.reserve("a", 17)
+    assert c.block_table("a") == [0, 1] and c.free_pages() == 6
+    c.advance("a", 17)
+    c.reserve("a", 15)  # fills page 1 exactly
+    assert len(c.block_table("a")) == 2
+    c.advance("a", 15)
+    c.reserve("a", 1)
+    assert len(c.block_table("a")) == 3
+    assert c.write_slots("a", 0, 30, 3).tolist() == [1 * 16 + 14, 1 * 16 + 15, 2 * 16 + 0]
+    c.check()
+    with pytest.raises(RuntimeError, match="without reserved pages"):
+        c.advance("a", 40)
+
+
+def test_freed_pages_are_used_again_last_freed_first():
+    c = CacheManager(16, [4], [None], n_slots=3)
+    for r in "ab":
+        c.admit(r)
+        c.reserve(r, 32)
+        c.advance(r, 32)
+    assert c.free_pages() == 0
+    c.admit("c")
+    with pytest.raises(OutOfPages, match="needs 1 more pages in cache group 0, 0 are free"):
+        c.reserve("c", 1)
+    assert c.block_table("c") == []  # all or nothing
+    pages_a = c.block_table("a")
+    c.release("a")
+    c.reserve("c", 20)
+    assert sorted(c.block_table("c")) == sorted(pages_a)
+    assert c.block_table("c")[0] == pages_a[-1]  # the page freed last is on top
+    c.check()
+    with pytest.raises(KeyError):
+        c.release("a")  # freed twice
+
+
+def test_slots():
+    c = CacheManager(16, [4], [None], n_slots=2)
+    s = {c.admit("a"), c.admit("b")}
+    assert s == {0, 1}
+    with pytest.raises(OutOfSlots):
+        c.admit("c")
+    with pytest.raises(KeyError, match="already live"):
+        c.admit("a")
+    c.release("a")
+    assert c.admit("c") in s
+    c.check()
+
+
+def test_window_group_gives_pages_back():
+    # group 0 keeps all keys, group 1 a window of 20 tokens
+    c = CacheManager(8, [32, 32], [None, 20], n_slots=1)
+    c.admit("a")
+    n = 0
+    for step in [5, 30, 1, 1, 17, 2, 64, 1]:
+        c.reserve("a", step)
+        # during the step the first new token at position n still reads keys n-19 .. n
+        lo = max(0, n - 20 + 1) // 8
+        assert all(p != RELEASED for p in c.block_table("a", 1)[lo:])
+        c.advance("a", step)
+        n += step
+        c.check()
+        tbl = c.block_table("a", 1)
+        first_needed = max(0, n - 20 + 1) // 8
+        assert all(p == RELEASED for p in tbl[:first_needed]) and all(p != RELEASED for p in tbl[first_needed:])
+        assert RELEASED not in c.block_table("a", 0)
+    assert c.free_pages(1) == 32 - sum(p != RELEASED for p in c.block_table("a", 1))
+    assert c.free_pages(1) > c.free_pages(0)
+    c.release("a")
+    assert c.free_pages(0) == c.free_pages(1) == 32
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
+    rng = random.Random(seed)
+    c = CacheManager(16, [24, 24], [None, 40], n_slots=5)
+    live, n_next = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            rid = f"r{n_next}"
+            n_next += 1
+            c.admit(rid)
+            live[rid] = 0
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 7, 16, 33])
+            if c.can_reserve(rid, n):
+                c.reserve(rid, n)
+                c.advance(rid, n)
+                live[rid] += n
+                assert c.length(rid) == live[rid]
+            else:
+                with pytest.raises(OutOfPages):
+                    c.reserve(rid, n)
+        elif live:
+            rid = rng.choice(list(live))
+            c.release(rid)
+            del live[rid]
+        c.check()
+        held = {p for r in live for p in c.block_table(r, 0)}
+        assert len(held) + c.free_pages(0) == 24
+    for rid in list(live):
+        c.release(rid)
+    c.check()
+    assert c.free_pages(0) == c.free_pages(1) == 24 and c.free_slots() == 5
+
+
+# ---------------------------------------------------------------- scheduler
+def fake_token(req, pos):
+    return (hash((req.rid, pos)) % 97) + 3
+
+
+def drive(sched, max_steps=10_000):
+    """Run the scheduler to the end with the stand-in model; returns the plans."""
+    plans = []
+    for _ in range(max_steps):
+        if not sched.has_work():
+            break
+        plan = sched.plan()
+        sched.finished.clear()
+        if not plan:
+            continue
+        assert sum(e.n for e in plan) <= sched.max_step_tokens
+        assert len({e.request.rid for e in plan}) == len(plan)
+        for e in plan:
+            assert e.start == e.request.n_fed == sched.cache.length(e.request.rid)
+            assert e.wants_logits == (e.start + e.n == e.request.n_known())
+            sched.cache.advance(e.request.rid, e.n)
+        sched.cache.check()
+        plans.append([(e.request.rid, e.start, e.n, e.wants_logits) for e in plan])
+        sched.commit(plan, [fake_token(e.request, e.start + e.n) for e in plan if e.wants_logits])
+    else:
+        raise AssertionError("the scheduler did not finish")
+    return plans
+
+
+def mk(cache_pages=64, page=16, max_batch=4, budget=24, max_seq=None):
+    c = CacheManager(page, [cache_pages], [None], n_slots=max_batch)
+    return Scheduler(c, max_batch, budget, max_seq)
+
+
+def test_budget_decodes_first_then_prompt_portions():
+    s = mk(budget=24)
+    reqs = [Request(i, list(range(n)), max_new=4) for i, n in enumerate([5, 17, 33])]
+    for r in reqs:
+        s.add(r)
+    plans = drive(s)
+    # step 0: 5 + 17 + the first 2 of request 2 = 24 tokens
+    assert plans[0] == [(0, 0, 5, True), (1, 0, 17, True), (2, 0, 2, False)]
+    # step 1: requests 0 and 1 decode one token each, request 2 gets the other 22
+    assert plans[1] == [(0, 5, 1, True), (1, 17, 1, True), (2, 2, 22, False)]
+    assert plans[2] == [(0, 6, 1, True), (1, 18, 1, True), (2, 24, 9, True)]
+    for r in reqs:
+        assert len(r.generated) == 4 and r.finish_reason == "length"
+        assert r.generated == [fake_token(r, len(r.prompt) + i) for i in range(4)]
+    assert s.cache.live_requests() == [] and s.cache.free_pages() == 64
+
+
+def test_cut_on_a_prompt_end_and_prompt_of_one():
+    """A budget that ends exactly on a prompt's end (fastgen/generate.py:815-817
+    holds one token back there; here the portion simply ends the prompt and
+    asks for its logits) and a prompt of one token."""
+    s = mk(budget=8)
+    a, b = Request("a", list(range(8)), 2), Request("b", [7], 3)
+    s.add(a), s.add(b)
+    plans = drive(s)
+    assert plans[0] == [("a", 0, 8, True)]
+    assert plans[1] == [("a", 8, 1, True), ("b", 0, 1, True)]
+    assert len(a.generated) == 2 and len(b.generated) == 3
+
+
+def test_max_batch_and_first_come_first_served():
+    s = mk(max_batch=2, budget=64)
+    reqs = [Request(i, [1] * 10, max_new=3 + i) for i in range(4)]
+    for r in reqs:
+        s.add(r)
+    plans = drive(s)
+    for p in plans:
+        assert len(p) <= 2
+    first_seen = {}
+    for i, p in enumerate(plans):
+        for rid, *_ in p:
+            first_seen.setdefault(rid, i)
+    assert first_seen[0] == first_seen[1] == 0 and first_seen[2] <= first_seen[3]
+    assert first_seen[2] == 3  # as soon as request 0 (3 new tokens) has ended
+
+
+def test_stop_ids_and_caps():
+    s = mk(max_seq=20)
+    r = Request("a", [1, 2, 3], max_new=50)
+    stop_at = fake_token(r, 3 + 4)
+    r.stop_ids = (stop_at,)
+    s.add(r)
+    drive(s)
+    assert r.finish_reason == "stop" and r.generated[-1] == stop_at and len(r.generated) <= 5
+    r2 = Request("b", [1, 2, 3], max_new=50)
+    s.add(r2)
+    drive(s)
+    assert r2.finish_reason == "max_seq" and r2.n_known() == 20
+    with pytest.raises(ValueError, match="can never fit"):
+        s.add(Request("c", [0] * 20, 1))
+    with pytest.raises(ValueError, match="empty prompt"):
+        s.add(Request("d", [], 1))
+
+
+def test_out_of_pages_preempts_the_youngest_and_recomputes():
+    # 6 pages of 16: three requests of 30 tokens fill them; growing needs a 7th page
+    s = mk(cache_pages=6, max_batch=3, budget=64)
+    reqs = [Request(i, [i] * 30, max_new=8) for i in range(3)]
+    for r in reqs:
+        s.add(r)
+    plans = drive(s)
+    assert s.n_preemptions >= 1
+    assert reqs[2].preemptions >= 1 and reqs[0].preemptions == 0  # the youngest gives way, the oldest never
+    # the preempted request is fed again from its first token, generated tokens included
+    refeeds = [p for plan in plans for p in plan if p[0] == 2 and p[1] == 0]
+    assert len(refeeds) == 1 + reqs[2].preemptions
+    for r in reqs:
+        assert r.generated == [fake_token(r, 30 + i) for i in range(8)]  # same tokens as without preemption
+    assert s.cache.free_pages() == 6
+
+
+def test_alone_and_out_of_pages_ends_with_cache_full():
+    s = mk(cache_pages=2, max_batch=1, budget=64, max_seq=1000)
+    r = Request("a", [1] * 20, max_new=100)
+    s.add(r)
+    drive(s)
+    assert r.finish_reason in ("cache_full", "max_seq") and r.n_known() <= 32
+
+
+def test_waiting_request_is_not_admitted_without_room_for_its_prompt():
+    s = mk(cache_pages=4, max_batch=4, budget=64)
+    a, b = Request("a", [1] * 40, 4), Request("b", [2] * 40, 4)
+    s.add(a), s.add(b)
+    plans = drive(s)
+    assert [p[0] for p in plans[0]] == ["a"]  # b's 41 tokens need 3 pages, 1 is free
+    assert b.preemptions == 0 and len(b.generated) == 4
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_load_finishes_with_the_right_tokens(seed):
+    rng = random.Random(seed)
+    s = mk(cache_pages=rng.choice([8, 12, 40]), page=16, max_batch=rng.choice([2, 4, 8]), budget=rng.choice([8, 24, 100]))
+    s.cache.n_slots  # noqa: B018
+    reqs = [Request(i, [rng.randrange(50) for _ in range(rng.choice([1, 3, 20, 45, 90]))], max_new=rng.choice([1, 5, 30]))
+            for i in range(12)]
+    for r in reqs:
+        s.add(r)
+    drive(s)
+    for r in reqs:
+        assert r.finish_reason == "length" and r.generated == [fake_token(r, len(r.prompt) + i) for i in range(r.max_new)]

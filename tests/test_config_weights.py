@@ -1,0 +1,182 @@
+"""Configuration, registry, layout and weight errors (no GPU)."""
+
+import json
+
+import pytest
+import torch
+
+from plain_llama import TINY_A, TINY_B, plain_random_weights, plain_rope_frequencies, plain_rope_shuffle
+
+from fastgen_amd.config import (
+    ConfigError, ModelArgs, ModelLayout, PartSpec, RunEntry, LayerSpec, get_architecture, read_config_json,
+    registered_architectures,
+)
+from fastgen_amd.engine.model import build_parts
+from fastgen_amd.parts import build_part
+from fastgen_amd.weights import (
+    DictSource, RandomSource, SafetensorsSource, WeightError, check_against_specs, write_model_folder,
+)
+
+
+def test_typed_config_from_hf_keys():
+    a = ModelArgs.from_hf_config(TINY_B)
+    assert (a.dim, a.ffn_dim, a.n_layers, a.n_heads, a.n_kv_heads, a.head_dim) == (192, 512, 3, 6, 3, 32)
+    assert (a.norm_eps, a.vocab_size, a.tie_embeddings, a.max_position) == (1e-5, 384, False, 256)
+    assert a.rope.scaled and (a.rope.theta, a.rope.factor, a.rope.original_context) == (500000.0, 8.0, 64)
+    b = ModelArgs.from_hf_config(TINY_A)
+    assert not b.rope.scaled and b.tie_embeddings and b.head_dim == 16
+    # kv heads default to the heads (fastgen/utils/loading.py:64-67)
+    c = ModelArgs.from_hf_config({k: v for k, v in TINY_A.items() if k != "num_key_value_heads"})
+    assert c.n_kv_heads == c.n_heads
+    # round trip through config.json keys
+    assert ModelArgs.from_hf_config(a.to_hf_config()) == a
+
+
+@pytest.mark.parametrize("key", ["hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
+                                 "rms_norm_eps", "vocab_size", "rope_theta"])
+def test_missing_key_is_named(key):
+    cfg = {k: v for k, v in TINY_B.items() if k != key}
+    with pytest.raises(ConfigError, match=key):
+        ModelArgs.from_hf_config(cfg)
+
+
+def test_config_refusals():
+    with pytest.raises(ConfigError, match="rope_type"):
+        ModelArgs.from_hf_config(dict(TINY_B, rope_scaling=dict(TINY_B["rope_scaling"], rope_type="yarn")))
+    with pytest.raises(ConfigError, match="low_freq_factor"):
+        sc = {k: v for k, v in TINY_B["rope_scaling"].items() if k != "low_freq_factor"}
+        ModelArgs.from_hf_config(dict(TINY_B, rope_scaling=sc))
+    with pytest.raises(ConfigError, match="head_dim"):
+        ModelArgs.from_hf_config(dict(TINY_B, head_dim=64))
+    with pytest.raises(ConfigError, match="multiple"):
+        ModelArgs.from_hf_config(dict(TINY_B, num_key_value_heads=4))
+    with pytest.raises(ConfigError, match="attention_bias"):
+        ModelArgs.from_hf_config(dict(TINY_B, attention_bias=True))
+
+
+def test_registry():
+    assert "LlamaForCausalLM" in registered_architectures()
+    assert get_architecture(TINY_A).name == "LlamaForCausalLM"
+    with pytest.raises(ConfigError, match="Unsupported model type 'GPT2LMHeadModel'"):
+        get_architecture({"architectures": ["GPT2LMHeadModel"]})
+
+
+def test_layout_is_data():
+    arch = get_architecture(TINY_B)
+    lay = arch.layout(arch.parse(TINY_B))
+    assert len(lay.layers) == 3 and [e.layer for e in lay.order] == [0, 1, 2]
+    assert lay.layers[1].mixer.kind == "attention" and lay.layers[1].ffn.kind == "swiglu"
+    assert lay.layers[2].mixer.options["n_kv_heads"] == 3 and lay.layers[0].ffn.options["hidden_dim"] == 512
+    assert lay.head.options["tied_to"] is None
+    # the order may name a layer twice and let an entry read an earlier entry's cache
+    twice = ModelLayout(lay.dim, lay.vocab_size, lay.embed, lay.layers,
+                        (RunEntry(0), RunEntry(1), RunEntry(1), RunEntry(2, reads_cache_of=0)), lay.final_norm, lay.head)
+    assert len(twice.order) == 4
+    with pytest.raises(ValueError, match="does not run before"):
+        ModelLayout(lay.dim, lay.vocab_size, lay.embed, lay.layers, (RunEntry(0, reads_cache_of=1), RunEntry(1)),
+                    lay.final_norm, lay.head)
+    with pytest.raises(ValueError, match="does not exist"):
+        ModelLayout(lay.dim, lay.vocab_size, lay.embed, lay.layers, (RunEntry(7),), lay.final_norm, lay.head)
+    with pytest.raises(KeyError, match="no mixer of kind 'nonesuch'"):
+        build_part("mixer", PartSpec("nonesuch"))
+
+
+def test_rope_part_matches_the_plain_formulas():
+    arch = get_architecture(TINY_B)
+    lay = arch.layout(arch.parse(TINY_B))
+    rope = build_part("position", lay.layers[0].mixer.options["position"])
+    assert torch.equal(rope.frequencies(), plain_rope_frequencies(32, 500000.0, TINY_B["rope_scaling"]))
+    w = torch.randn(6 * 32, 20)
+    assert torch.equal(rope.arrange_rows(w, 6), plain_rope_shuffle(w, 6))
+    # a partial rotation permutes the rotary part of each head only
+    part = build_part("position", PartSpec("rope", options=dict(head_dim=8, rotary_dim=4, theta=100.0)))
+    rows = torch.arange(16.0)[:, None]
+    assert part.arrange_rows(rows, 2)[:, 0].tolist() == [0, 2, 1, 3, 4, 5, 6, 7, 8, 10, 9, 11, 12, 13, 14, 15]
+    assert part.frequencies().tolist() == pytest.approx([1.0, 0.1])
+
+
+def _specs(cfg):
+    arch = get_architecture(cfg)
+    return build_parts(arch.layout(arch.parse(cfg))).tensor_specs()
+
+
+def test_tensor_names_are_the_checkpoint_names():
+    for cfg in (TINY_A, TINY_B):
+        names = {s.name: s.shape for s in _specs(cfg)}
+        plain = plain_random_weights(cfg, 0)
+        assert names == {k: tuple(v.shape) for k, v in plain.items()}
+
+
+def test_one_error_lists_everything_wrong():
+    w = plain_random_weights(TINY_B, 0)
+    del w["model.layers.1.mlp.up_proj.weight"], w["model.norm.weight"]
+    w["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(192)
+    w["model.layers.2.self_attn.k_proj.weight"] = torch.zeros(96, 100)
+    with pytest.raises(WeightError) as e:
+        check_against_specs(DictSource(w), _specs(TINY_B))
+    msg = str(e.value)
+    assert "missing tensors (2): model.layers.1.mlp.up_proj.weight, model.norm.weight" in msg
+    assert "unexpected tensors (1): model.layers.0.self_attn.q_proj.bias" in msg
+    assert "model.layers.2.self_attn.k_proj.weight is [96, 100], expected [96, 192]" in msg
+
+
+def test_tied_head_in_the_file():
+    w = plain_random_weights(TINY_A, 0)
+    specs = _specs(TINY_A)
+    arch = get_architecture(TINY_A)
+    dup = build_parts(arch.layout(arch.parse(TINY_A))).duplicates()
+    w["lm_head.weight"] = w["model.embed_tokens.weight"].clone()
+    check_against_specs(DictSource(w), specs, dup)  # an equal copy is tolerated
+    w["lm_head.weight"] = w["lm_head.weight"] + 1
+    with pytest.raises(WeightError, match="unexpected tensors .*lm_head.weight"):
+        check_against_specs(DictSource(w), specs, dup)
+
+
+def test_random_weights_folder(tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    folder = write_model_folder(tmp_path / "m", TINY_B, seed=5)
+    cfg = read_config_json(folder)
+    assert ModelArgs.from_hf_config(cfg) == ModelArgs.from_hf_config(TINY_B)
+    src = SafetensorsSource(folder)
+    check_against_specs(src, _specs(TINY_B))
+    t = load_file(str(folder / "model.safetensors"))
+    assert t["model.layers.0.mlp.down_proj.weight"].dtype == torch.float32
+    assert abs(float(t["model.embed_tokens.weight"].std()) - 0.02) < 2e-3
+    assert abs(float(t["model.norm.weight"].mean()) - 1) < 5e-3 and float(t["model.norm.weight"].std()) < 0.02
+    # the same seed gives the same tensors, another seed others; a tensor does not depend on the rest
+    again = write_model_folder(tmp_path / "m2", TINY_B, seed=5)
+    other = write_model_folder(tmp_path / "m3", TINY_B, seed=6)
+    t2, t3 = load_file(str(again / "model.safetensors")), load_file(str(other / "model.safetensors"))
+    assert all(torch.equal(t[k], t2[k]) for k in t) and not torch.equal(t["lm_head.weight"], t3["lm_head.weight"])
+    one = RandomSource([s for s in _specs(TINY_B) if s.name == "lm_head.weight"], 5)
+    assert torch.equal(one.get("lm_head.weight"), t["lm_head.weight"])
+    bf = write_model_folder(tmp_path / "m4", TINY_A, seed=5, dtype=torch.bfloat16)
+    assert load_file(str(bf / "model.safetensors"))["model.norm.weight"].dtype == torch.bfloat16
+    # sharded folders with an index are read by name too
+    sh = tmp_path / "sharded"
+    sh.mkdir()
+    keys = sorted(t)
+    save_file({k: t[k] for k in keys[::2]}, str(sh / "model-00001-of-00002.safetensors"))
+    save_file({k: t[k] for k in keys[1::2]}, str(sh / "model-00002-of-00002.safetensors"))
+    json.dump({"weight_map": {k: f"model-0000{1 + i % 2}-of-00002.safetensors" for i, k in enumerate(keys)}},
+              open(sh / "model.safetensors.index.json", "w"))
+    s2 = SafetensorsSource(sh)
+    assert sorted(s2.names()) == keys and torch.equal(s2.get(keys[3]), t[keys[3]])
+    (sh / "model.safetensors.index.json").unlink()
+    assert sorted(SafetensorsSource(sh).names()) == keys
+    with pytest.raises(WeightError, match="no model.safetensors"):
+        SafetensorsSource(tmp_path)
+    with pytest.raises(ConfigError, match="not a model folder"):
+        read_config_json(tmp_path)
+
+
+def test_dtype_policy():
+    from fastgen_amd.parts import MATRIX, VECTOR, TABLE_INT, place
+
+    m32, m16 = torch.randn(4, 4), torch.randn(4, 4).bfloat16()
+    assert place(m32, MATRIX, torch.bfloat16, "cpu").dtype == torch.bfloat16
+    assert place(m16, MATRIX, torch.float32, "cpu").dtype == torch.float32
+    assert place(torch.randn(4), VECTOR, torch.bfloat16, "cpu").dtype == torch.float32  # stored in 32-bit: stays
+    assert place(torch.randn(4).bfloat16(), VECTOR, torch.bfloat16, "cpu").dtype == torch.bfloat16
+    assert place(torch.arange(4), TABLE_INT, torch.bfloat16, "cpu").dtype == torch.int32

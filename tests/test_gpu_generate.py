@@ -1,0 +1,161 @@
+"""Generation through the entry points: greedy against the plain
+implementation, sampling with seeds, preemption, the reference-style
+interface and the command line."""
+
+import json
+import queue
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from helpers import save_model_folder
+from plain_llama import TINY_A, TINY_B, plain_forward, plain_greedy, plain_random_weights
+
+pytestmark = pytest.mark.gpu
+REPO = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def tiny_b(tmp_path_factory):
+    w = plain_random_weights(TINY_B, 1)
+    w = {k: v * 8 if ("q_proj" in k or "k_proj" in k or "lm_head" in k) else v for k, v in w.items()}
+    folder = save_model_folder(tmp_path_factory.mktemp("genB"), TINY_B, w)
+    g = torch.Generator().manual_seed(9)
+    prompts = [torch.randint(0, 384, (n,), generator=g).tolist() for n in (1, 12, 40, 90, 150)]
+    return dict(folder=folder, weights=w, prompts=prompts)
+
+
+def test_greedy_generation_matches_the_plain_implementation(tiny_b):
+    """BASELINE's second workload: prompts of 1, 12, 40, 90 and 150 tokens, 16
+    new tokens each, portions of at most 24 tokens a step beside decodes."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=1024, max_batch=4,
+                             max_step_tokens=24)
+    got = eng.generate(tiny_b["prompts"], SamplingParams(temperature=0.0, max_new_tokens=16))
+    want = [plain_greedy(tiny_b["weights"], TINY_B, p, 16) for p in tiny_b["prompts"]]
+    assert got == want
+    assert eng.runner.cache.live_requests() == []
+    eng.runner.cache.check()
+
+
+def test_preemption_gives_the_same_tokens(tiny_b):
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    prompts = tiny_b["prompts"][1:4]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=40)
+    roomy = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=16, max_tokens=1024, max_batch=3,
+                               max_step_tokens=64)
+    want = roomy.generate(prompts, sp)
+    # 12+40+90 prompt tokens and 120 new ones in 15 pages of 16: not all fit at once
+    tight = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=16, max_tokens=240, max_batch=3,
+                               max_step_tokens=64)
+    got = tight.generate(prompts, sp)
+    assert tight.scheduler.n_preemptions > 0
+    assert got == want
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_temperature_sampling_is_seeded_and_independent_of_the_batch(tiny_b, dtype):
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    mk = lambda budget, mb: Engine.from_folder(tiny_b["folder"], dtype, page_size=32, max_tokens=1024, max_batch=mb,
+                                               max_step_tokens=budget)
+    sps = [SamplingParams(temperature=0.8, top_p=0.95, seed=100 + i, max_new_tokens=16) for i in range(5)]
+    together = mk(24, 4).generate(tiny_b["prompts"], sps)
+    again = mk(24, 4).generate(tiny_b["prompts"], sps)
+    assert together == again
+    if dtype == torch.float32:
+        alone = [mk(512, 1).generate([p], [sp])[0] for p, sp in zip(tiny_b["prompts"], sps)]
+        assert together == alone  # neither batch-mates nor the cut of the prompt change a request's draw
+    other = mk(24, 4).generate(tiny_b["prompts"], [SamplingParams(temperature=0.8, top_p=0.95, seed=7 + i,
+                                                                  max_new_tokens=16) for i in range(5)])
+    assert other != together
+    greedy = mk(24, 4).generate(tiny_b["prompts"], SamplingParams(temperature=0.0, max_new_tokens=16))
+    assert greedy != together
+
+
+def test_sampled_tokens_follow_the_models_distribution(tiny_b):
+    """The first sampled token of one prompt under many seeds against
+    softmax(logits / T) of the plain implementation."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    prompt = tiny_b["prompts"][2]
+    probs = torch.softmax(plain_forward(tiny_b["weights"], TINY_B, prompt)[-1] / 0.7, -1)
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=64 * 64, max_batch=64,
+                             max_step_tokens=4096)
+    n = 2048
+    counts = torch.zeros(384)
+    for s0 in range(0, n, 64):
+        outs = eng.generate([prompt] * 64, [SamplingParams(temperature=0.7, seed=1 + s0 + i, max_new_tokens=1)
+                                            for i in range(64)])
+        for o in outs:
+            counts[o[0]] += 1
+    big = probs * n >= 5
+    chi2 = (((counts - n * probs) ** 2 / (n * probs))[big]).sum()
+    assert chi2 < 2.0 * int(big.sum()) + 30, (float(chi2), int(big.sum()))
+
+
+def test_stop_ids_and_logprobs(tiny_b):
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=512, max_batch=2)
+    prompt = tiny_b["prompts"][1]
+    free = plain_greedy(tiny_b["weights"], TINY_B, prompt, 10)
+    rid = eng.add_request(prompt, SamplingParams(max_new_tokens=10, stop_ids=(free[4],), logprobs=True))
+    done = []
+    while eng.has_work():
+        done += eng.step()
+    assert done[0].rid == rid and done[0].finish_reason == "stop"
+    stop_at = free.index(free[4])
+    assert done[0].generated == free[: stop_at + 1]  # ends with the stop token
+    toks = prompt + done[0].generated
+    lp = torch.log_softmax(plain_forward(tiny_b["weights"], TINY_B, toks), -1)
+    want = [float(lp[len(prompt) - 1 + i, t]) for i, t in enumerate(done[0].generated)]
+    assert done[0].logprobs == pytest.approx(want, abs=1e-4)
+
+
+def test_reference_style_interface(tiny_b):
+    from fastgen_amd.generate import Fastgen, GenArgs, Packet
+
+    fg = Fastgen.build(tiny_b["folder"], GenArgs(use_sampling=False, max_batch=3, max_seq=1024, max_gen=8,
+                                                cache_block=32, max_prefill=48, dtype=torch.float32), stop_tokens=())
+    q = queue.Queue()
+    for i, p in enumerate(tiny_b["prompts"]):
+        q.put(Packet(thread_id=f"t{i}", tokens=p, max_gen=5 if i == 0 else None))
+    q.put(None)
+    out = {pkt.thread_id: pkt.tokens for pkt in fg.generate(q)}
+    assert set(out) == {f"t{i}" for i in range(5)}
+    for i, p in enumerate(tiny_b["prompts"]):
+        assert out[f"t{i}"] == plain_greedy(tiny_b["weights"], TINY_B, p, 5 if i == 0 else 8)
+    # sizing from a memory budget (fastgen/utils/tune.py:68-84)
+    fg2 = Fastgen.build(tiny_b["folder"], GenArgs(gpu_gb=0.6, prefill_gb=0.5, dtype=torch.bfloat16))
+    per_token = 2 * 3 * 32 * 2 * 3
+    assert fg2.engine.scheduler.max_seq == pytest.approx((0.1e9 - fg2.engine.model.weight_bytes()) / per_token, abs=64)
+
+
+def test_command_line(tiny_b):
+    prompt = tiny_b["prompts"][1]
+    cmd = [sys.executable, str(REPO / "bin" / "fgchat"), str(tiny_b["folder"]), "--prompt-ids",
+           ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0", "--dtype", "float32",
+           "--max-seq", "256", "--gpu-gb", "1"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(x) for x in proc.stdout.strip().splitlines()[0].split(",")]
+    assert got == plain_greedy(tiny_b["weights"], TINY_B, prompt, 6)
+    assert "tok/s" in proc.stderr
+
+
+def test_smoke_entry():
+    sys.path.insert(0, str(REPO))
+    import __graft_entry__
+
+    __graft_entry__.smoke()

@@ -1,0 +1,316 @@
+"""Each part alone against its plain formula, models whose layers differ, run
+orders that name a layer twice or share a cache, and a toy mixer with state
+of its own that is registered, built and stepped from this file alone."""
+
+import json
+from typing import Any, Mapping, Optional
+
+import pytest
+import torch
+
+import traces
+from helpers import assert_close, run_trace
+from plain_llama import (
+    plain_attention, plain_rmsnorm, plain_rope_frequencies, plain_rope_interleaved, plain_rope_shuffle, plain_swiglu,
+)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tol(dtype):
+    return dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_feed_forward_embedding_head_alone(dtype):
+    from fastgen_amd.config import PartSpec
+    from fastgen_amd.parts import build_part
+
+    torch.manual_seed(0)
+    D, F, V, T = 72, 200, 131, 9
+    norm = build_part("norm", PartSpec("rmsnorm", "n", dict(dim=D, eps=1e-3)))
+    w = 1 + 0.1 * torch.randn(D)
+    norm.load({"n.weight": w}, dtype, DEV)
+    assert norm.weight.dtype == torch.float32  # stored in 32-bit: stays so
+    h, delta = torch.randn(T, D), torch.randn(T, D).to(dtype)
+    hd = h.to(DEV)
+    y = norm.forward(hd, delta.to(DEV), dtype).cpu()
+    assert torch.allclose(y.float(), plain_rmsnorm(h + delta.float(), w, 1e-3).to(dtype).float(), **_tol(dtype))
+    assert torch.equal(hd.cpu(), h + delta.float())
+
+    ffn = build_part("feed_forward", PartSpec("swiglu", "m", dict(dim=D, hidden_dim=F)))
+    ws = {f"m.{k}_proj.weight": torch.randn(*s) * 0.2 for k, s in (("gate", (F, D)), ("up", (F, D)), ("down", (D, F)))}
+    ws = {k: v.to(dtype).float() for k, v in ws.items()}
+    ffn.load(ws, dtype, DEV)
+    x = torch.randn(T, D).to(dtype)
+    got = ffn.forward(x.to(DEV)).cpu().float()
+    want = plain_swiglu(x.float(), ws["m.gate_proj.weight"], ws["m.up_proj.weight"], ws["m.down_proj.weight"])
+    assert torch.allclose(got, want, **_tol(dtype))
+
+    emb = build_part("embedding", PartSpec("embedding", "e", dict(vocab_size=V, dim=D)))
+    table = torch.randn(V, D).to(dtype)
+    emb.load({"e.weight": table}, dtype, DEV)
+    tok = torch.tensor([0, V - 1, 5, 5], dtype=torch.int32)
+    assert torch.equal(emb.forward(tok.to(DEV)).cpu(), table[tok.long()].float())
+
+    head = build_part("head", PartSpec("lm_head", "lm_head", dict(vocab_size=V, dim=D, tied_to="e")))
+    assert head.tensor_specs() == []
+    head.tie(emb.weight)
+    logits = head.forward(x.to(DEV))
+    assert logits.dtype == torch.float32 and logits.shape == (T, V)
+    assert torch.allclose(logits.cpu(), x.float() @ table.float().T, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,KV,hd,rot,window", [(6, 2, 32, 32, None), (5, 5, 16, 8, None), (4, 1, 48, 48, 21),
+                                               (2, 2, 64, 0, None)])
+def test_attention_mixer_alone(dtype, H, KV, hd, rot, window):
+    """The mixer with its own cache, two sequences in two steps, against the
+    plain attention over whole sequences; rotary_dim < head_dim and no
+    rotation at all are other position encodings of the same mixer."""
+    from fastgen_amd.cache import CacheManager
+    from fastgen_amd.cache.storage import CacheStorage, group_entries
+    from fastgen_amd.config import PartSpec
+    from fastgen_amd.engine import StepEntry, build_context
+    from fastgen_amd.parts import build_part
+
+    torch.manual_seed(1)
+    D, P = 40, 16
+    pos_spec = PartSpec("rope", options=dict(head_dim=hd, rotary_dim=rot, theta=1000.0)) if rot else PartSpec("none")
+    mixer = build_part("mixer", PartSpec("attention", "a", dict(
+        dim=D, n_heads=H, n_kv_heads=KV, head_dim=hd, scale=hd**-0.5, window=window, position=pos_spec)))
+    ws = {f"a.{k}_proj.weight": (torch.randn(*s) * 0.3).to(dtype).float()
+          for k, s in (("q", (H * hd, D)), ("k", (KV * hd, D)), ("v", (KV * hd, D)), ("o", (D, H * hd)))}
+    mixer.load(ws, dtype, DEV)
+    need = mixer.paged_need()
+    assert (need.n_kv_heads, need.head_dim, need.window) == (KV, hd, window)
+    groups = group_entries([need])
+    cache = CacheManager(P, [16], [window], n_slots=2)
+    storage = CacheStorage(groups, [16], P, {}, 2, dtype, DEV)
+    store = storage.store_for(0)
+    lens = {"x": 45, "y": 20}
+    xs = {r: torch.randn(n, D).to(dtype) for r, n in lens.items()}
+    outs = {r: [] for r in lens}
+    for r in lens:
+        cache.admit(r)
+    for cuts in ({"x": (0, 30), "y": (0, 1)}, {"x": (30, 45), "y": (1, 20)}):
+        entries = [StepEntry(r, [0] * (b - a), []) for r, (a, b) in cuts.items()]
+        for e in entries:
+            cache.reserve(e.rid, len(e.tokens))
+        ctx = build_context(entries, cache, dtype, DEV)
+        x = torch.cat([xs[r][a:b] for r, (a, b) in cuts.items()]).to(DEV)
+        y = mixer.forward(x, ctx, store).cpu()
+        at = 0
+        for r, (a, b) in cuts.items():
+            outs[r].append(y[at : at + b - a])
+            at += b - a
+            cache.advance(r, b - a)
+    f = plain_rope_frequencies(rot, 1000.0) if rot else None
+    for r, n in lens.items():
+        x = xs[r].float()
+        q = (x @ ws["a.q_proj.weight"].T).view(n, H, hd)
+        k = (x @ ws["a.k_proj.weight"].T).view(n, KV, hd)
+        v = (x @ ws["a.v_proj.weight"].T).view(n, KV, hd)
+        if rot:
+            # checkpoint order rotates pairs (i, i + rot/2) of the rotary part
+            def rope(t, nh):
+                perm = plain_rope_shuffle(torch.eye(nh * rot), nh)  # row permutation as a matrix
+                tr = t[..., :rot].reshape(n, nh * rot) @ perm.T
+                tr = plain_rope_interleaved(tr.view(n, nh, rot), torch.arange(n), f)
+                return torch.cat([tr, t[..., rot:]], -1)
+            q, k = rope(q, H), rope(k, KV)
+        want = plain_attention(q, k, v, window).reshape(n, H * hd) @ ws["a.o_proj.weight"].T
+        assert torch.allclose(torch.cat(outs[r]).float(), want, **_tol(dtype)), r
+
+
+# ------------------------------------------------- layers that differ; order
+class _HybridArch:
+    """A test-only architecture: per layer its own head counts, window and
+    feed-forward width, and a run order given in the configuration."""
+
+    name = "HybridTestModel"
+
+    def parse(self, config: Mapping[str, Any]):
+        return dict(config)
+
+    def to_hf_config(self, args):
+        return dict(args)
+
+    def layout(self, a):
+        from fastgen_amd.config import LayerSpec, ModelLayout, PartSpec, RunEntry
+
+        D = a["dim"]
+        norm = lambda p: PartSpec("rmsnorm", p, dict(dim=D, eps=a["eps"]))
+        layers = []
+        for i, l in enumerate(a["layers"]):
+            p = f"blocks.{i}"
+            if l["mixer"] == "attention":
+                pos = PartSpec("rope", options=dict(head_dim=l["hd"], rotary_dim=l.get("rot", l["hd"]), theta=a["theta"]))
+                mixer = PartSpec("attention", f"{p}.attn", dict(dim=D, n_heads=l["H"], n_kv_heads=l["KV"],
+                                                               head_dim=l["hd"], scale=l["hd"] ** -0.5,
+                                                               window=l.get("window"), position=pos))
+            else:
+                mixer = PartSpec(l["mixer"], f"{p}.mix", dict(dim=D, decay=l["decay"]))
+            layers.append(LayerSpec(mixer, PartSpec("swiglu", f"{p}.ffn", dict(dim=D, hidden_dim=l["F"])),
+                                    norm(f"{p}.n1"), norm(f"{p}.n2")))
+        order = tuple(RunEntry(o[0], o[1]) for o in a["order"])
+        return ModelLayout(D, a["vocab"], PartSpec("embedding", "emb", dict(vocab_size=a["vocab"], dim=D)),
+                           tuple(layers), order, norm("final"),
+                           PartSpec("lm_head", "head", dict(vocab_size=a["vocab"], dim=D, tied_to=None)))
+
+
+def _plain_hybrid(w, a, tokens, mixers):
+    """Plain whole-sequence forward of the hybrid model; attention entries
+    that read another entry's cache use that entry's rotated k and v."""
+    T = len(tokens)
+    h = w["emb.weight"][torch.tensor(tokens)]
+    kv_of = {}
+    for idx, (li, src) in enumerate(a["order"]):
+        l, p = a["layers"][li], f"blocks.{li}"
+        x = plain_rmsnorm(h, w[f"{p}.n1.weight"], a["eps"])
+        if l["mixer"] == "attention":
+            H, KV, hd, rot = l["H"], l["KV"], l["hd"], l.get("rot", l["hd"])
+            f = plain_rope_frequencies(rot, a["theta"])
+
+            def rope(t, nh):
+                perm = plain_rope_shuffle(torch.eye(nh * rot), nh)
+                tr = t[..., :rot].reshape(T, nh * rot) @ perm.T
+                tr = plain_rope_interleaved(tr.view(T, nh, rot), torch.arange(T), f)
+                return torch.cat([tr, t[..., rot:]], -1)
+
+            q = rope((x @ w[f"{p}.attn.q_proj.weight"].T).view(T, H, hd), H)
+            if src is None:
+                k = rope((x @ w[f"{p}.attn.k_proj.weight"].T).view(T, KV, hd), KV)
+                v = (x @ w[f"{p}.attn.v_proj.weight"].T).view(T, KV, hd)
+                kv_of[idx] = (k, v)
+            else:
+                k, v = kv_of[src]
+            m = plain_attention(q, k, v, l.get("window")).reshape(T, H * hd) @ w[f"{p}.attn.o_proj.weight"].T
+        else:
+            m = mixers[l["mixer"]](x, w, p, l)
+        h = h + m
+        x = plain_rmsnorm(h, w[f"{p}.n2.weight"], a["eps"])
+        h = h + plain_swiglu(x, w[f"{p}.ffn.gate_proj.weight"], w[f"{p}.ffn.up_proj.weight"],
+                             w[f"{p}.ffn.down_proj.weight"])
+    return plain_rmsnorm(h, w["final.weight"], a["eps"]) @ w["head.weight"].T
+
+
+def _hybrid_case(tmp_path, args, seed=3, sharpen=8.0):
+    from safetensors.torch import load_file, save_file
+
+    from fastgen_amd.weights import write_model_folder
+
+    folder = write_model_folder(tmp_path / "hybrid", dict(args, architectures=["HybridTestModel"]), seed=seed)
+    w = load_file(str(folder / "model.safetensors"))
+    w = {k: (v * sharpen if ("q_proj" in k or "k_proj" in k) else v).to(torch.bfloat16).float() for k, v in w.items()}
+    save_file(w, str(folder / "model.safetensors"))
+    return folder, w
+
+
+@pytest.fixture
+def hybrid_arch():
+    from fastgen_amd.config import register_architecture, unregister_architecture
+
+    register_architecture(_HybridArch(), replace=True)
+    yield
+    unregister_architecture("HybridTestModel")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layers_differ_and_order_is_data(tmp_path, hybrid_arch, dtype):
+    """Three layers with different head counts, head sizes, windows and
+    widths; the order runs layer 1 twice and lets the last entry read the
+    first entry's cache.  Two cache groups arise (window and no window)."""
+    from fastgen_amd.engine import Model, ModelRunner
+
+    args = dict(dim=96, vocab=211, eps=2e-6, theta=5000.0, layers=[
+        dict(mixer="attention", H=4, KV=2, hd=16, F=136),
+        dict(mixer="attention", H=3, KV=1, hd=32, rot=16, window=24, F=72),
+        dict(mixer="attention", H=8, KV=2, hd=16, F=200),
+    ], order=[(0, None), (1, None), (1, None), (2, 0)])
+    folder, w = _hybrid_case(tmp_path, args)
+    model = Model.from_folder(folder, dtype, DEV)
+    runner = ModelRunner(model, page_size=16, max_tokens=512, max_requests=4)
+    assert len(runner.groups) == 2 and sorted(len(g.entries) for g in runner.groups) == [1, 2]
+    lengths = {"a": 70, "b": 33, "c": 5}
+    g = torch.Generator().manual_seed(4)
+    toks = {r: torch.randint(0, 211, (n,), generator=g).tolist() for r, n in lengths.items()}
+    want = {r: _plain_hybrid(w, args, t, {}) for r, t in toks.items()}
+    noise = {r: want[r] + (want[r].abs().max() * 4e-3) for r in want}  # bf16: 0.8% of the largest logit
+    for tr in (traces.whole(lengths), traces.chunks(lengths), traces.mixed(lengths, seed=2)):
+        got = run_trace(runner, tr, toks)
+        assert_close(got, want, dtype, noise, "hybrid")
+        # the window group gives pages back while the request is still live
+    assert runner.cache.free_pages(0) == runner.cache.free_pages(1) == 32
+
+
+# ------------------------------------------------------ a toy mixer with state
+def _register_toy():
+    from fastgen_amd.parts import Mixer, StateNeed, TensorSpec, place, register_part
+
+    class ToyEma(Mixer):
+        """out_t = W s_t with s_t = decay * s_{t-1} + x_t, s kept per request
+        in a state slot of fixed size.  Plain torch on the device: a toy."""
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.dim, self.decay = spec.options["dim"], spec.options["decay"]
+
+        def tensor_specs(self):
+            return [TensorSpec(self._name("w.weight"), (self.dim, self.dim))]
+
+        def load(self, tensors, dtype, device):
+            self.w = place(tensors[self._name("w.weight")], "matrix", dtype, device)
+
+        def state_need(self):
+            return StateNeed((self.dim,), torch.float32)
+
+        def forward(self, x, ctx, store):
+            out = torch.empty_like(x)
+            at = 0
+            for b in range(ctx.n_seqs):
+                s = store.state[int(ctx.slot_ids_host[b])]
+                for t in range(at, at + int(ctx.q_lens[b])):
+                    s.mul_(self.decay).add_(x[t].float())
+                    out[t] = (self.w.float() @ s).to(x.dtype)
+                at += int(ctx.q_lens[b])
+            return out
+
+    register_part("mixer", "toy_ema", ToyEma, replace=True)
+
+
+def _plain_toy(x, w, p, l):
+    s, out = torch.zeros(x.shape[1]), []
+    for t in range(x.shape[0]):
+        s = l["decay"] * s + x[t]
+        out.append(w[f"{p}.mix.w.weight"] @ s)
+    return torch.stack(out)
+
+
+def test_toy_mixer_with_state_of_its_own(tmp_path, hybrid_arch):
+    from fastgen_amd.engine import Model, ModelRunner, StepEntry
+    from fastgen_amd.parts import unregister_part
+
+    _register_toy()
+    try:
+        args = dict(dim=48, vocab=97, eps=1e-5, theta=100.0, layers=[
+            dict(mixer="toy_ema", decay=0.9, F=64),
+            dict(mixer="attention", H=3, KV=3, hd=16, F=80),
+            dict(mixer="toy_ema", decay=0.5, F=64),
+        ], order=[(0, None), (1, None), (2, None)])
+        folder, w = _hybrid_case(tmp_path, args)
+        model = Model.from_folder(folder, torch.float32, DEV)
+        assert sorted(model.state_needs()) == [0, 2]
+        runner = ModelRunner(model, page_size=16, max_tokens=256, max_requests=2)
+        assert len(runner.groups) == 1 and runner.storage.state[0].shape == (2, 48)
+        lengths = {"a": 37, "b": 20, "c": 9}
+        g = torch.Generator().manual_seed(5)
+        toks = {r: torch.randint(0, 97, (n,), generator=g).tolist() for r, n in lengths.items()}
+        want = {r: _plain_hybrid(w, args, t, {"toy_ema": _plain_toy}) for r, t in toks.items()}
+        # two live at a time: c takes a slot that a or b left, and finds it cleared
+        got = run_trace(runner, traces.mixed(lengths, max_live=2, seed=1), toks)
+        assert_close(got, want, torch.float32, None, "toy")
+        assert runner.cache.free_slots() == 2
+    finally:
+        unregister_part("mixer", "toy_ema")
