@@ -139,7 +139,9 @@ def test_reference_style_interface(tiny_b):
     # sizing from a memory budget (fastgen/utils/tune.py:68-84)
     fg2 = Fastgen.build(tiny_b["folder"], GenArgs(gpu_gb=0.6, prefill_gb=0.5, dtype=torch.bfloat16))
     per_token = 2 * 3 * 32 * 2 * 3
-    assert fg2.engine.scheduler.max_seq == pytest.approx((0.1e9 - fg2.engine.model.weight_bytes()) / per_token, abs=64)
+    pool = fg2.engine.runner.cache.n_pages[0] * 64
+    assert pool == pytest.approx((0.1e9 - fg2.engine.model.weight_bytes()) / per_token, abs=64)
+    assert fg2.engine.scheduler.max_seq == 256  # one request is capped by max_position_embeddings
 
 
 def test_command_line(tiny_b):
