@@ -13,6 +13,7 @@
 // fp32, o = P.V; query head h reads kv head h / (H/KV).  With window > 0 only
 // keys p-window+1..p are seen.
 #include "common.h"
+#include "kv_layout.h"
 
 #define ATT_WAVES 4
 #define ATT_TILE 64
@@ -58,6 +59,8 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
   const int pos = positions[t];
   const int* table = block_table + (size_t)seq * bt_stride;
   const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const KvLayout lay(page_size, hd);
+  const size_t head_elems = (size_t)page_size * hd;
 
   const T* qrow = q + (size_t)t * q_stride + (size_t)h * hd;
   float* qs = q_s[wave];
@@ -78,12 +81,12 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
     float s = -INFINITY;
     if (valid) {
       const int page = table[key / page_size];
-      const T* krow =
-          k_pages + (((size_t)page * n_kv + kvh) * page_size + key % page_size) * hd;
+      const T* khead = k_pages + ((size_t)page * n_kv + kvh) * head_elems;
+      const int kappa = key % page_size;
       float acc = 0.f;
       for (int d = 0; d < hd; d += 8) {
         Vec8<T> kv;
-        kv.load(krow + d);
+        kv.load(khead + lay.k_off(kappa, d));
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc += qs[d + e] * kv.v[e];
       }
@@ -99,26 +102,29 @@ __global__ __launch_bounds__(ATT_WAVES* FG_WAVE) void paged_attention_general_ke
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < MAXD; ++i) o[i] *= alpha;
-    // ---- o += P.V: lane owns head dims lane, lane+64, ...; eight keys at a
-    // time, which lie in one page because pages hold a multiple of 8 keys
-    for (int j8 = 0; j8 < ATT_TILE; j8 += 8) {
-      const int k0 = kb + j8;
-      if (k0 > pos) break;
-      if (k0 + 7 < first) continue;
-      const int page = table[k0 / page_size];
-      const int off = k0 % page_size;
+    // ---- o += P.V: lane owns head dims lane, lane+64, ...; one stored chunk
+    // of eight key slots at a time (one page; with the permuted order the
+    // slots of chunk g of a 32-key group are keys 4g..4g+3 and 16+4g..16+4g+3)
+    for (int q = 0; q < ATT_TILE / 8; ++q) {
+      const int base = lay.permuted ? kb + 32 * (q / 4) + 4 * (q % 4) : kb + 8 * q;  // lowest key of the chunk
+      const int stride_hi = lay.permuted ? 12 : 0;  // slots 4..7 are 16 keys on (4 + 12)
+      if (base > pos) { if (lay.permuted) continue; else break; }
+      if (base + 7 + stride_hi < first) continue;
+      const int page = table[base / page_size];
+      const T* vhead = v_pages + ((size_t)page * n_kv + kvh) * head_elems;
+      const int kc = lay.v_slot(base % page_size) / 8;
 #pragma unroll
       for (int i = 0; i < MAXD; ++i) {
         const int d = lane + i * FG_WAVE;
         if (d < hd) {
           Vec8<T> vv;
-          vv.load(v_pages + (((size_t)page * n_kv + kvh) * hd + d) * page_size + off);
+          vv.load(vhead + lay.v_chunk_off(kc, d));
           float acc = o[i];
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const int kk = k0 + e;
+            const int kk = base + e + (e >= 4 ? stride_hi : 0);
             // select, not multiply: a slot never written may hold NaN
-            if (kk >= first && kk <= pos) acc += ps[j8 + e] * vv.v[e];
+            if (kk >= first && kk <= pos) acc += ps[kk - kb] * vv.v[e];
           }
           o[i] = acc;
         }

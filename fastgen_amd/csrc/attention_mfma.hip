@@ -1,0 +1,486 @@
+// Paged causal attention on the matrix cores (bf16 in, fp32 accumulate) for
+// gfx950.  Compiled once per head size: -DFG_HD=<multiple of 16, at most 256>.
+//
+// Both kernels work on *items*: an item is a run of consecutive query tokens
+// of one sequence; its rows are (token, query head of one kv head's group),
+// token-major.  Per 64-key tile a wave computes, with v_mfma_f32_16x16x32_bf16,
+//   S^T = K Q^T      (A = 16 keys x 32 head dims, B = Q^T, 16 query rows)
+//   O^T += V^T P^T   (A = 16 head dims x 32 keys of the transposed V page)
+// so that every lane keeps ONE query row (lane % 16) in both results: the
+// running maximum, the sum and the rescaling need no exchange but two
+// shuffles across the four lane groups.  The 64 keys of a tile are assigned
+// to S's rows so that the probabilities a lane group ends up holding are 8
+// consecutive key *slots* of the value page (kv_layout.h), which makes V's
+// operand one 16-byte read and lets P stay in registers.  With the chunked
+// page layout every operand load of a wave is 1 KB of contiguous memory.
+//
+//  * fg_attn_split (decode and very short portions, <= 16 rows an item): the
+//    key range of an item is cut into splits (grid.x) and a split's tiles are
+//    dealt to the 4 waves, which stream K and V straight from the pages;
+//    partial (max, sum, O) go to scratch and fg_attn_combine merges them.
+//  * fg_attn_tile (prompt portions, 64 rows an item): K and V tiles are staged
+//    in LDS and shared by 4 waves of 16 rows each.
+//
+// Semantics as in attention.hip (fastgen/forward.py:176-258).
+#include "common.h"
+#include "kv_layout.h"
+
+#ifndef FG_HD
+#error "compile with -DFG_HD=<head size>"
+#endif
+static_assert(FG_HD % 16 == 0 && FG_HD >= 16 && FG_HD <= 256, "head size: multiple of 16 up to 256");
+
+constexpr int HD = FG_HD;
+constexpr int NKS = (HD + 31) / 32;  // 32-wide steps over the head dimension (last may be half)
+constexpr int NDB = HD / 16;         // 16-wide blocks of the head dimension
+constexpr int TILE = 64;             // keys per tile
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// key (within a tile) of S^T row `row` (0..15) of key block kb (0..3)
+__device__ __forceinline__ int key_of(int kb, int row) { return 16 * kb + row; }
+
+// An item: a run of consecutive query tokens of one sequence.
+struct Item {
+  int seq, tok0, n_tok, pos0;  // sequence, flat index and position of its first token
+};
+__device__ __forceinline__ Item load_item(const int* items, int i) {
+  const int4 v = *(const int4*)(items + 4 * i);
+  return Item{v.x, v.y, v.z, v.w};
+}
+
+// page lookup without a division when the page size is a power of two
+struct Pager {
+  const int* table;
+  int page_size, shift;
+  __device__ __forceinline__ int page_of(int key) const {
+    return table[shift >= 0 ? key >> shift : key / page_size];
+  }
+  __device__ __forceinline__ int in_page(int key) const {
+    return shift >= 0 ? key & (page_size - 1) : key % page_size;
+  }
+};
+
+struct ItemRows {
+  int pos;    // position of this lane's query row, -1 for a padding row
+  int first;  // first key the row sees
+};
+
+// One 64-key tile for one wave, operands given by loader functors.
+//   load_k(kb, ks) -> bf16x8 : K[16*kb + lane%16][32*ks + 8*(lane/16) ..+7]
+//   load_v(db, ks) -> bf16x8 : V^T[16*db + lane%16][the 8 keys 32*ks + 4g + i, 32*ks + 16 + 4g + i]
+//                              with g = lane/16, i = 0..3: the keys of pop[ks]
+template <class LK, class LV>
+__device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf16x8 (&qop)[NKS], float scale,
+                                            float& m, float& l, f32x4 (&o)[NDB], LK load_k, LV load_v) {
+  const int g = (threadIdx.x % FG_WAVE) >> 4;
+  f32x4 s[4];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb) {
+    s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks)
+      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_k(kb, ks), qop[ks], s[kb], 0, 0, 0);
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = k0 + key_of(kb, 4 * g + i);
+      const float v = (key >= me.first && key <= me.pos) ? s[kb][i] * scale : -INFINITY;
+      s[kb][i] = v;
+      mx = fmaxf(mx, v);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, FG_WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, FG_WAVE));
+  const float m_new = fmaxf(m, mx);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+  const float alpha = __expf(m - m_use);                 // m = -inf: 0
+  float sum = 0.f;
+  bf16x8 pop[2];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = __expf(s[kb][i] - m_use);
+      sum += p;
+      pop[kb >> 1][4 * (kb & 1) + i] = (__bf16)p;
+    }
+  l = l * alpha + sum;  // this lane's share of the row's sum; the groups are added at the end
+  m = m_new;
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) {
+    o[db] *= alpha;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_v(db, ks), pop[ks], o[db], 0, 0, 0);
+  }
+}
+
+// Q^T operand: lane holds Q[row lane%16][32*ks + 8*(lane/16) ..+7]
+__device__ __forceinline__ void load_q(bf16x8 (&qop)[NKS], const bf16_t* qrow /* null: padding row */) {
+  const int g = (threadIdx.x % FG_WAVE) >> 4;
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    const int d = 32 * ks + 8 * g;
+    qop[ks] = (qrow && d < HD) ? *(const bf16x8*)(qrow + d) : zero8();
+  }
+}
+
+// ------------------------------------------------------------------ split
+// grid (n_splits, n_kv, n_items), 256 threads.  items: [n_items][4] = sequence,
+// flat index of the first token, number of tokens, position of the first
+// token; n_tok * (H / KV) <= 16.
+__global__ __launch_bounds__(256) void attn_split_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int n_heads, int n_kv, int page_size,
+    int page_shift, float scale, int window) {
+  __shared__ float o_s[2][16][HD + 1];
+  __shared__ float ml_s[2][16][2];
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int split = blockIdx.x, n_splits = gridDim.x, kvh = blockIdx.y, item = blockIdx.z;
+  const int G = n_heads / n_kv;
+  const Item it = load_item(items, item);
+  const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
+  const KvLayout lay(page_size, HD);
+
+  const int pos_last = it.pos0 + it.n_tok - 1;
+  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+  ItemRows me{-1, 0};
+  const bf16_t* qrow = nullptr;
+  if (r16 < it.n_tok * G) {
+    me.pos = it.pos0 + r16 / G;
+    me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
+    qrow = q + (size_t)(it.tok0 + r16 / G) * q_stride + (size_t)(kvh * G + r16 % G) * HD;
+  }
+  bf16x8 qop[NKS];
+  load_q(qop, qrow);
+
+  const int t_lo = first_min / TILE, t_hi = pos_last / TILE;
+  const int per_split = (t_hi - t_lo + 1 + n_splits - 1) / n_splits;
+  const int t_begin = t_lo + split * per_split;
+  const int t_end = min(t_hi + 1, t_begin + per_split);
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const size_t head_elems = (size_t)page_size * HD;  // elements of one kv head in a page
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const int k0 = t * TILE;
+    // K chunks of this lane: key 16*kb + r16 of the tile, head dims 32*ks + 8*g
+    const bf16_t* kptr[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const int key = k0 + 16 * kb + r16;
+      kptr[kb] = nullptr;
+      if (key >= first_min && key <= pos_last)
+        kptr[kb] = k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                   lay.k_off(pager.in_page(key), 8 * g);
+    }
+    // V chunks of this lane: keys 32*ks + 4*g + (0..3) and 16 more on; head dim 16*db + r16
+    const bf16_t* vptr[2][2];
+    bool vedge[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int ka = k0 + 32 * ks + 4 * g, kb2 = ka + 16;
+      vedge[ks] = ka < first_min || kb2 + 3 > pos_last;
+      vptr[ks][0] = vptr[ks][1] = nullptr;
+      if (ka + 3 >= first_min && ka <= pos_last)
+        vptr[ks][0] = v_pages + ((size_t)pager.page_of(ka) * n_kv + kvh) * head_elems +
+                      lay.v_off(pager.in_page(ka), r16);
+      if (!lay.permuted && kb2 + 3 >= first_min && kb2 <= pos_last)
+        vptr[ks][1] = v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
+                      lay.v_off(pager.in_page(kb2), r16);
+      if (lay.permuted && !vptr[ks][0] && kb2 + 3 >= first_min && kb2 <= pos_last)
+        // the first half lies outside the range but the second inside: same chunk, same page
+        vptr[ks][0] = v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
+                      lay.v_off(pager.in_page(kb2), r16) - 4;
+    }
+    const size_t k_step = (size_t)4 * lay.kb * 8;       // 32 head dims on: 4 chunks of kb keys
+    const size_t v_step = (size_t)(page_size / 8) * 128;  // 16 head dims on: one dim block
+    auto load_k = [&](int kb, int ks) -> bf16x8 {
+      return (kptr[kb] && 32 * ks + 8 * g < HD) ? *(const bf16x8*)(kptr[kb] + ks * k_step) : zero8();
+    };
+    auto load_v = [&](int db, int ks) -> bf16x8 {
+      bf16x8 v = zero8();
+      if (lay.permuted) {
+        if (vptr[ks][0]) v = *(const bf16x8*)(vptr[ks][0] + db * v_step);
+      } else {
+        bf16x4 lo = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f}, hi = lo;
+        if (vptr[ks][0]) lo = *(const bf16x4*)(vptr[ks][0] + db * v_step);
+        if (vptr[ks][1]) hi = *(const bf16x4*)(vptr[ks][1] + db * v_step);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = lo[e];
+          v[4 + e] = hi[e];
+        }
+      }
+      if (vedge[ks]) {  // keys outside the item's range may hold anything, NaN included
+        const int ka = k0 + 32 * ks + 4 * g;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int kk = ka + (e & 3) + 16 * (e >> 2);
+          if (kk < first_min || kk > pos_last) v[e] = (__bf16)0.f;
+        }
+      }
+      return v;
+    };
+    attend_tile(k0, me, qop, scale, m, l, o, load_k, load_v);
+  }
+  l += __shfl_xor(l, 16, FG_WAVE);
+  l += __shfl_xor(l, 32, FG_WAVE);
+
+  // ---- merge the 4 waves pairwise in registers: 2,3 -> 0,1 then 1 -> 0
+  auto put = [&](int slot) {
+    if (g == 0) {
+      ml_s[slot][r16][0] = m;
+      ml_s[slot][r16][1] = l;
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o_s[slot][r16][16 * db + 4 * g + i] = o[db][i];
+  };
+  auto take = [&](int slot) {
+    const float mo = ml_s[slot][r16][0], lo = ml_s[slot][r16][1];
+    const float M = fmaxf(m, mo);
+    const float fs = m == -INFINITY ? 0.f : __expf(m - M);
+    const float fo = mo == -INFINITY ? 0.f : __expf(mo - M);
+    l = fs * l + fo * lo;
+    m = M;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] = fs * o[db][i] + fo * o_s[slot][r16][16 * db + 4 * g + i];
+  };
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  take(0);
+  if (r16 >= it.n_tok * G) return;
+  const int t_out = it.tok0 + r16 / G, h_out = kvh * G + r16 % G;
+  if (n_splits == 1) {
+    bf16_t* orow = out + (size_t)t_out * out_stride + (size_t)h_out * HD;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[db][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v;
+    }
+  } else {
+    const size_t row = (((size_t)item * n_kv + kvh) * n_splits + split) * 16 + r16;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) *(f32x4*)(part_o + row * HD + 16 * db + 4 * g) = o[db];
+    if (g == 0) {
+      part_ml[row * 2] = m;
+      part_ml[row * 2 + 1] = l;
+    }
+  }
+}
+
+// grid (16 rows, n_kv, n_items), one thread per head dimension
+__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    const int* __restrict__ items, bf16_t* __restrict__ out, int out_stride,
+                                    int n_heads, int n_kv, int n_splits) {
+  const int r = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z, d = threadIdx.x;
+  const int G = n_heads / n_kv;
+  const Item it = load_item(items, item);
+  if (r >= it.n_tok * G || d >= HD) return;
+  const size_t row0 = (((size_t)item * n_kv + kvh) * n_splits) * 16 + r;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(row0 + (size_t)s * 16) * 2]);
+  float L = 0.f, O = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const size_t row = row0 + (size_t)s * 16;
+    const float ms = part_ml[row * 2];
+    const float f = ms == -INFINITY ? 0.f : __expf(ms - M);
+    L += f * part_ml[row * 2 + 1];
+    O += f * part_o[row * HD + d];
+  }
+  const int t = it.tok0 + r / G, h = kvh * G + r % G;
+  out[(size_t)t * out_stride + (size_t)h * HD + d] = (bf16_t)(O / L);
+}
+
+static int page_shift_of(int page_size) {
+  for (int s = 3; s < 31; ++s)
+    if ((1 << s) == page_size) return s;
+  return -1;
+}
+
+// part_o: fp32 [n_items * n_kv * n_splits * 16 * HD], part_ml: the same rows x 2;
+// both may be null when n_splits == 1.
+extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                             const void* v_pages, const int* block_table, int bt_stride, const int* items,
+                             int n_items, float* part_o, float* part_ml, int n_splits, int n_heads, int n_kv,
+                             int hd, int page_size, float scale, int window, hipStream_t stream) {
+  if (n_items <= 0) return FG_OK;
+  if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
+      n_splits < 1 || n_splits > 65535 || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
+      out_stride % 4 || (n_splits > 1 && (!part_o || !part_ml)))
+    return FG_ERR_ARG;
+  attn_split_kernel<<<dim3(n_splits, n_kv, n_items), 256, 0, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
+      block_table, bt_stride, items, part_o, part_ml, n_heads, n_kv, page_size, page_shift_of(page_size), scale,
+      window);
+  if (n_splits > 1)
+    attn_combine_kernel<<<dim3(16, n_kv, n_items), HD < 64 ? 64 : HD, 0, stream>>>(
+        part_o, part_ml, items, (bf16_t*)out, out_stride, n_heads, n_kv, n_splits);
+  return fg_launch_status();
+}
+
+// ------------------------------------------------------------------- tile
+// grid (n_items, n_kv), 256 threads: 4 waves of 16 rows; an item has at most
+// 64 / (H / KV) tokens.  The K and V tiles go through LDS in the order the
+// operands are read: K [4 key blocks][HD/8 chunks][16 keys][8], V [HD/16 dim
+// blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
+__global__ __launch_bounds__(256) void attn_tile_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
+    int page_size, int page_shift, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) bf16_t k_s[TILE * HD];
+  __shared__ __attribute__((aligned(16))) bf16_t v_s[TILE * HD];
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int item = blockIdx.x, kvh = blockIdx.y;
+  const int G = n_heads / n_kv;
+  const Item it = load_item(items, item);
+  const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
+  const KvLayout lay(page_size, HD);
+  const int pos_last = it.pos0 + it.n_tok - 1;
+  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+
+  const int row = wave * 16 + r16;
+  ItemRows me{-1, 0};
+  const bf16_t* qrow = nullptr;
+  if (row < it.n_tok * G) {
+    me.pos = it.pos0 + row / G;
+    me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
+    qrow = q + (size_t)(it.tok0 + row / G) * q_stride + (size_t)(kvh * G + row % G) * HD;
+  }
+  bf16x8 qop[NKS];
+  load_q(qop, qrow);
+  // the keys this wave's rows can see: tiles outside are skipped by the wave
+  int w_hi = me.pos, w_lo = me.pos < 0 ? 0x7fffffff : me.first;
+#pragma unroll
+  for (int msk = 1; msk < 16; msk <<= 1) {
+    w_hi = max(w_hi, __shfl_xor(w_hi, msk, FG_WAVE));
+    w_lo = min(w_lo, __shfl_xor(w_lo, msk, FG_WAVE));
+  }
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const size_t head_elems = (size_t)page_size * HD;
+  constexpr int KCH = HD / 8;  // 16-byte chunks in a key
+  for (int k0 = (first_min / TILE) * TILE; k0 <= pos_last; k0 += TILE) {
+    __syncthreads();  // the previous tile is no longer read
+    // K: chunk (block kb, dims 8c.., key r) -> k_s[((kb*KCH + c)*16 + r)*8]; r fastest over threads
+    for (int w = threadIdx.x; w < TILE * KCH; w += 256) {
+      const int r = w & 15, c = (w >> 4) % KCH, kb = (w >> 4) / KCH, key = k0 + 16 * kb + r;
+      bf16x8 v = zero8();
+      if (key >= first_min && key <= pos_last)
+        v = *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                             lay.k_off(pager.in_page(key), 8 * c));
+      *(bf16x8*)(k_s + (size_t)w * 8) = v;
+    }
+    // V: chunk (dim block db, key chunk kc = 4*ks + gg, dim r) -> v_s[((db*8 + kc)*16 + r)*8];
+    // its slots are keys 32*ks + 4*gg + (0..3) and 16 more on
+    for (int w = threadIdx.x; w < NDB * 8 * 16; w += 256) {
+      const int r = w & 15, kc = (w >> 4) & 7, db = w >> 7;
+      const int ka = k0 + 32 * (kc >> 2) + 4 * (kc & 3), kb2 = ka + 16;
+      bf16x8 v = zero8();
+      const bool in_a = ka + 3 >= first_min && ka <= pos_last, in_b = kb2 + 3 >= first_min && kb2 <= pos_last;
+      if (lay.permuted) {
+        if (in_a || in_b) {
+          const int kk = in_a ? ka : kb2;
+          v = *(const bf16x8*)(v_pages + ((size_t)pager.page_of(kk) * n_kv + kvh) * head_elems +
+                               lay.v_off(pager.in_page(kk), 16 * db + r) - (in_a ? 0 : 4));
+        }
+      } else {
+        bf16x4 lo = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f}, hi = lo;
+        if (in_a)
+          lo = *(const bf16x4*)(v_pages + ((size_t)pager.page_of(ka) * n_kv + kvh) * head_elems +
+                                lay.v_off(pager.in_page(ka), 16 * db + r));
+        if (in_b)
+          hi = *(const bf16x4*)(v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
+                                lay.v_off(pager.in_page(kb2), 16 * db + r));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = lo[e];
+          v[4 + e] = hi[e];
+        }
+      }
+      if (ka < first_min || kb2 + 3 > pos_last) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int kk = ka + (e & 3) + 16 * (e >> 2);
+          if (kk < first_min || kk > pos_last) v[e] = (__bf16)0.f;
+        }
+      }
+      *(bf16x8*)(v_s + (size_t)w * 8) = v;
+    }
+    __syncthreads();
+    if (k0 > w_hi || k0 + TILE <= w_lo) continue;  // nothing in this tile for this wave's rows
+    auto load_k = [&](int kb, int ks) -> bf16x8 {
+      const int c = 4 * ks + g;
+      return c < KCH ? *(const bf16x8*)(k_s + ((kb * KCH + c) * 16 + r16) * 8) : zero8();
+    };
+    auto load_v = [&](int db, int ks) -> bf16x8 {
+      return *(const bf16x8*)(v_s + ((db * 8 + 4 * ks + g) * 16 + r16) * 8);
+    };
+    attend_tile(k0, me, qop, scale, m, l, o, load_k, load_v);
+  }
+  l += __shfl_xor(l, 16, FG_WAVE);
+  l += __shfl_xor(l, 32, FG_WAVE);
+  if (row < it.n_tok * G) {
+    bf16_t* orow = out + (size_t)(it.tok0 + row / G) * out_stride + (size_t)(kvh * G + row % G) * HD;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[db][i] * inv);
+      *(bf16x4*)(orow + 16 * db + 4 * g) = v;
+    }
+  }
+}
+
+extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                            const void* v_pages, const int* block_table, int bt_stride, const int* items,
+                            int n_items, int n_heads, int n_kv, int hd, int page_size, float scale, int window,
+                            hipStream_t stream) {
+  if (n_items <= 0) return FG_OK;
+  if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 64 || page_size < 8 || page_size % 8 ||
+      n_kv > 65535 || window < 0 || q_stride % 8 || out_stride % 4)
+    return FG_ERR_ARG;
+  attn_tile_kernel<<<dim3(n_items, n_kv), 256, 0, stream>>>(
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
+      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window);
+  return fg_launch_status();
+}
+
+extern "C" int fg_attn_head_dim() { return HD; }

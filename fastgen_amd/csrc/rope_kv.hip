@@ -7,12 +7,13 @@
 //   x[2i] = a cos - b sin,  x[2i+1] = b cos + a sin,
 // rounded once at the store.  Pairs beyond rotary_dim are left as they are.
 //
-// Cache layout, per cache layer: K pages [n_pages, KV, P, hd] (a key's head
-// is hd contiguous elements), V pages [n_pages, KV, hd, P] (transposed: the
-// keys of a page are contiguous for one head dimension), so that both matrix
-// products of attention read 16 contiguous bytes per lane.  A token's place
-// is slot = page*P + offset; a negative slot means "write nothing".
+// Cache layout, per cache layer: K pages [n_pages, KV, P*hd], V pages
+// [n_pages, KV, hd*P], the elements inside a page ordered as kv_layout.h
+// says (16-byte chunks placed for the matrix-core kernels; V transposed).  A
+// token's place is slot = page*P + offset; a negative slot means "write
+// nothing".
 #include "common.h"
+#include "kv_layout.h"
 
 #define ROPE_THREADS 256
 
@@ -29,6 +30,8 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
   const int slot = write_kv ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot % page_size : 0;
+  const KvLayout lay(page_size, hd);
+  const size_t head_elems = (size_t)page_size * hd;
 
   // q heads then k heads: (n_heads + n_kv) * hd/2 pairs
   const int n_rot_heads = n_heads + (write_kv ? n_kv : 0);
@@ -50,7 +53,7 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
       x[1] = from_f<T>(b);
     } else if (slot >= 0) {
       const int kvh = head - n_heads;
-      T* dst = k_pages + (((size_t)page * n_kv + kvh) * page_size + off) * hd + 2 * i;
+      T* dst = k_pages + ((size_t)page * n_kv + kvh) * head_elems + lay.k_off(off, 2 * i);
       dst[0] = from_f<T>(a);
       dst[1] = from_f<T>(b);
     }
@@ -59,7 +62,57 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
     const T* v = row + (size_t)(n_heads + n_kv) * hd;
     for (int e = threadIdx.x; e < n_kv * hd; e += ROPE_THREADS) {
       const int kvh = e / hd, d = e % hd;
-      v_pages[(((size_t)page * n_kv + kvh) * hd + d) * page_size + off] = v[e];
+      v_pages[((size_t)page * n_kv + kvh) * head_elems + lay.v_off(off, d)] = v[e];
+    }
+  }
+}
+
+// The same with eight consecutive elements (four pairs) a thread; for
+// hd % 8 == 0, rotary_dim % 8 == 0 and rows 16-byte aligned.
+template <class T>
+__global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
+    T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
+    const float* __restrict__ freqs, const int* __restrict__ slots, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
+    int write_kv) {
+  const int t = blockIdx.x;
+  T* row = qkv + (size_t)t * row_stride;
+  const float pos = (float)positions[t];
+  const int slot = write_kv ? slots[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  const KvLayout lay(page_size, hd);
+  const size_t head_elems = (size_t)page_size * hd;
+  const int cph = hd / 8;  // chunks per head
+  const int n_rot = (n_heads + (write_kv ? n_kv : 0)) * cph;
+  const int n_v = slot >= 0 ? n_kv * cph : 0;
+  for (int w = threadIdx.x; w < n_rot + n_v; w += ROPE_THREADS) {
+    if (w < n_rot) {
+      const int head = w / cph, c = w % cph;
+      if (head >= n_heads && slot < 0) continue;
+      T* x = row + (size_t)head * hd + 8 * c;
+      float v[8];
+      load8<T>(x, v);
+      if (8 * c < rotary_dim) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float ang = pos * freqs[4 * c + j];
+          const float sn = sinf(ang), cs = cosf(ang);
+          const float a = v[2 * j], b = v[2 * j + 1];
+          v[2 * j] = a * cs - b * sn;
+          v[2 * j + 1] = b * cs + a * sn;
+        }
+      }
+      if (head < n_heads)
+        store8<T>(x, v);
+      else
+        store8<T>(k_pages + ((size_t)page * n_kv + (head - n_heads)) * head_elems + lay.k_off(off, 8 * c), v);
+    } else {
+      const int e = w - n_rot, kvh = e / cph, c = e % cph;
+      const T* src = row + (size_t)(n_heads + n_kv + kvh) * hd + 8 * c;
+      T* dst = v_pages + ((size_t)page * n_kv + kvh) * head_elems;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[lay.v_off(off, 8 * c + i)] = src[i];
     }
   }
 }
@@ -76,16 +129,20 @@ extern "C" int fg_rope_kv_write(void* qkv, int row_stride, const int* positions,
   if (hd <= 0 || hd % 2 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 ||
       page_size <= 0 || n_heads <= 0 || n_kv < 0)
     return FG_ERR_ARG;
+  if (write_kv && (hd % 8 || page_size % 8)) return FG_ERR_ARG;  // the page layout is in chunks of 8
   if (row_stride < (n_heads + (write_kv ? 2 * n_kv : 0)) * hd) return FG_ERR_ARG;
-  if (dtype == FG_F32)
-    rope_kv_write_kernel<float><<<n_tokens, ROPE_THREADS, 0, stream>>>(
-        (float*)qkv, row_stride, positions, freqs, slots, (float*)k_pages, (float*)v_pages,
-        n_heads, n_kv, hd, rotary_dim, page_size, write_kv);
-  else if (dtype == FG_BF16)
-    rope_kv_write_kernel<bf16_t><<<n_tokens, ROPE_THREADS, 0, stream>>>(
-        (bf16_t*)qkv, row_stride, positions, freqs, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
-        n_heads, n_kv, hd, rotary_dim, page_size, write_kv);
-  else
+  const bool vec = hd % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0;
+#define LAUNCH(T, KERNEL)                                                                         \
+  KERNEL<T><<<n_tokens, ROPE_THREADS, 0, stream>>>((T*)qkv, row_stride, positions, freqs, slots, \
+                                                   (T*)k_pages, (T*)v_pages, n_heads, n_kv, hd,  \
+                                                   rotary_dim, page_size, write_kv)
+  if (dtype == FG_F32) {
+    if (vec) LAUNCH(float, rope_kv_write_vec_kernel); else LAUNCH(float, rope_kv_write_kernel);
+  } else if (dtype == FG_BF16) {
+    if (vec) LAUNCH(bf16_t, rope_kv_write_vec_kernel); else LAUNCH(bf16_t, rope_kv_write_kernel);
+  } else {
     return FG_ERR_ARG;
+  }
+#undef LAUNCH
   return fg_launch_status();
 }

@@ -71,14 +71,83 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_kernel(
   }
 }
 
+// The same with each thread holding its share of the row in registers: 8
+// consecutive elements per 256-thread round, all loads of a round issued at
+// once.  For dim % 8 == 0 and dim <= 2048 * NIT.
+template <class TA, class TW, int NIT>
+__global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
+    float* __restrict__ h, const TA* __restrict__ delta, const TW* __restrict__ w,
+    TA* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* hrow = h + src * dim;
+  const TA* drow = delta ? delta + src * dim : nullptr;
+  float v[NIT][8];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
+    if (e < dim) load8<float>(hrow + e, v[it]);
+  }
+  if (drow) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
+      if (e < dim) {
+        float d[8];
+        load8<TA>(drow + e, d);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[it][i] += d[i];
+        if (!rows) store8<float>(hrow + e, v[it]);
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
+    if (e < dim) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss += v[it][i] * v[it][i];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss / (float)dim + eps);
+  TA* orow = out + (size_t)r * dim;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
+    if (e < dim) {
+      float wv[8], o[8];
+      load8<TW>(w + e, wv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = v[it][i] * rstd * wv[i];
+      store8<TA>(orow + e, o);
+    }
+  }
+}
+
+template <class TA, class TW>
+static void launch_add_rmsnorm(float* h, const void* delta, const void* w, void* out, const int* rows,
+                               int n_rows, int dim, float eps, hipStream_t stream) {
+#define VEC(NIT)                                                                              \
+  add_rmsnorm_vec_kernel<TA, TW, NIT><<<n_rows, ROWS_THREADS, 0, stream>>>(                   \
+      h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps)
+  if (dim % 8 == 0 && dim <= 2048) VEC(1);
+  else if (dim % 8 == 0 && dim <= 4096) VEC(2);
+  else if (dim % 8 == 0 && dim <= 8192) VEC(4);
+  else
+    add_rmsnorm_kernel<TA, TW><<<n_rows, ROWS_THREADS, 0, stream>>>(
+        h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps);
+#undef VEC
+}
+
 extern "C" int fg_add_rmsnorm(float* h, const void* delta, const void* w, void* out,
                               const int* rows, int n_rows, int dim, float eps, int act_dtype,
                               int w_dtype, hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
   if (dim <= 0) return FG_ERR_ARG;
-#define LAUNCH(TA, TW)                                                                       \
-  add_rmsnorm_kernel<TA, TW><<<n_rows, ROWS_THREADS, 0, stream>>>(                           \
-      h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps)
+#define LAUNCH(TA, TW) launch_add_rmsnorm<TA, TW>(h, delta, w, out, rows, n_rows, dim, eps, stream)
   if (act_dtype == FG_F32 && w_dtype == FG_F32) LAUNCH(float, float);
   else if (act_dtype == FG_BF16 && w_dtype == FG_BF16) LAUNCH(bf16_t, bf16_t);
   else if (act_dtype == FG_BF16 && w_dtype == FG_F32) LAUNCH(bf16_t, float);
@@ -140,6 +209,24 @@ __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_kernel(
   }
 }
 
+// eight elements a thread, for hidden % 8 == 0
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void silu_mul_vec_kernel(
+    const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
+  const TA* g = gu + (size_t)blockIdx.y * 2 * hidden;
+  const TA* u = g + hidden;
+  TA* o = out + (size_t)blockIdx.y * hidden;
+  const int e = (blockIdx.x * ROWS_THREADS + threadIdx.x) * 8;
+  if (e < hidden) {
+    float gv[8], uv[8], r[8];
+    load8<TA>(g + e, gv);
+    load8<TA>(u + e, uv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = gv[i] / (1.f + expf(-gv[i])) * uv[i];
+    store8<TA>(o + e, r);
+  }
+}
+
 extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, int act_dtype,
                            hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
@@ -147,15 +234,22 @@ extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, in
   // blockIdx.y is limited to 65535: rows beyond that go to further launches
   for (int r0 = 0; r0 < n_rows; r0 += 65535) {
     const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
-    dim3 grid((hidden + ROWS_THREADS - 1) / ROWS_THREADS, nr);
-    if (act_dtype == FG_F32)
-      silu_mul_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(
-          (const float*)gu + (size_t)r0 * 2 * hidden, (float*)out + (size_t)r0 * hidden, hidden);
-    else if (act_dtype == FG_BF16)
-      silu_mul_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(
-          (const bf16_t*)gu + (size_t)r0 * 2 * hidden, (bf16_t*)out + (size_t)r0 * hidden, hidden);
-    else
+    const bool vec = hidden % 8 == 0;
+    const int per_block = vec ? ROWS_THREADS * 8 : ROWS_THREADS;
+    dim3 grid((hidden + per_block - 1) / per_block, nr);
+    if (act_dtype == FG_F32) {
+      const float* g = (const float*)gu + (size_t)r0 * 2 * hidden;
+      float* o = (float*)out + (size_t)r0 * hidden;
+      if (vec) silu_mul_vec_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+      else silu_mul_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+    } else if (act_dtype == FG_BF16) {
+      const bf16_t* g = (const bf16_t*)gu + (size_t)r0 * 2 * hidden;
+      bf16_t* o = (bf16_t*)out + (size_t)r0 * hidden;
+      if (vec) silu_mul_vec_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+      else silu_mul_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+    } else {
       return FG_ERR_ARG;
+    }
   }
   return fg_launch_status();
 }

@@ -48,11 +48,18 @@ class StepContext:
     slot_ids: torch.Tensor  # int32 [B]: state slot of each sequence
     out_rows: torch.Tensor  # int32 [n_out]: flat token rows whose logits are wanted
     groups: List[GroupContext]
+    seq_records: Optional[torch.Tensor] = None  # int32 [B, 4]: sequence, first flat token, tokens, first position
     # host copies, for decisions about grids and kernels
     q_lens: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     n_cached: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
     slot_ids_host: np.ndarray = field(default_factory=lambda: np.zeros(0, np.int32))
+    q_start_host: np.ndarray = field(default_factory=lambda: np.zeros(1, np.int32))
     n_out: int = 0
+    # > 0: the context is the static one of a captured graph, replayed for requests of up to
+    # this many tokens; sizes derived from it must not depend on this step's lengths
+    graph_capacity: int = 0
+    # per-step derived data that kernels' dispatchers compute once and share between layers
+    scratch: dict = field(default_factory=dict)
 
     @property
     def max_q_len(self) -> int:
@@ -63,10 +70,12 @@ class StepContext:
         return int((self.q_lens + self.n_cached).max()) if self.n_seqs else 0
 
 
-def build_context(entries: Sequence[StepEntry], cache: CacheManager, act_dtype: torch.dtype,
-                  device: torch.device | str, vocab_size: Optional[int] = None) -> StepContext:
-    """Host vectors for ``entries`` (whose pages are already reserved), packed
-    into one int32 buffer and copied to the device once."""
+def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: Optional[int] = None,
+                 table_width: Optional[int] = None):
+    """Host side of :func:`build_context`: every int32 vector of the step in
+    one numpy buffer, and where each lies in it.  With ``table_width`` the block
+    tables have that many columns whatever the requests hold, so that steps of
+    the same batch shape have the same layout."""
     B = len(entries)
     q_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
     if B == 0 or (q_lens <= 0).any():
@@ -88,28 +97,53 @@ def build_context(entries: Sequence[StepEntry], cache: CacheManager, act_dtype: 
             out_rows.append(int(q_start[b]) + int(w))
     slot_ids = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
 
-    pieces = [tokens.astype(np.int32), positions, seq_of_token, q_start, (n_cached + q_lens).astype(np.int32),
-              slot_ids, np.asarray(out_rows, dtype=np.int32)]
-    tables = []
+    # one record per sequence (sequence, first flat token, tokens, first position): the items of the
+    # attention kernels when every sequence brings so few tokens that it is one item; first in the
+    # buffer, so 16-byte aligned
+    records = np.stack([np.arange(B, dtype=np.int32), q_start[:-1], q_lens, n_cached], axis=1).astype(np.int32)
+    pieces = [records.reshape(-1), tokens.astype(np.int32), positions, seq_of_token, q_start,
+              (n_cached + q_lens).astype(np.int32), slot_ids, np.asarray(out_rows, dtype=np.int32)]
+    table_shapes = []
     for g in range(cache.n_groups):
         width = max(cache.n_table_entries(e.rid, g) for e in entries)
+        if table_width is not None:
+            if width > table_width:
+                raise ValueError(f"a request holds {width} pages, the fixed table width is {table_width}")
+            width = table_width
         tbl = np.zeros((B, max(1, width)), dtype=np.int32)
         slots = np.empty(T, dtype=np.int32)
         for b, e in enumerate(entries):
             row = cache.block_table(e.rid, g)
             tbl[b, : len(row)] = row
             slots[q_start[b] : q_start[b + 1]] = cache.write_slots(e.rid, g, int(n_cached[b]), int(q_lens[b]))
-        tables.append(tbl.shape)
+        table_shapes.append(tbl.shape)
         pieces += [tbl.reshape(-1), slots]
-    packed = torch.from_numpy(np.concatenate(pieces)).to(device)
     offs = np.cumsum([0] + [p.size for p in pieces])
-    part = [packed[offs[i] : offs[i + 1]] for i in range(len(pieces))]
+    host = dict(q_lens=q_lens, n_cached=n_cached, slot_ids=slot_ids, q_start=q_start, n_out=len(out_rows))
+    return np.concatenate(pieces), offs, table_shapes, host
+
+
+def context_from_packed(packed: torch.Tensor, offs, table_shapes, host, page_size: int,
+                        act_dtype: torch.dtype) -> StepContext:
+    """Views into the device copy of a packed buffer."""
+    part = [packed[offs[i] : offs[i + 1]] for i in range(len(offs) - 1)]
     groups = [
-        GroupContext(cache.page_size, part[7 + 2 * g].view(tables[g]), part[8 + 2 * g])
-        for g in range(cache.n_groups)
+        GroupContext(page_size, part[8 + 2 * g].view(table_shapes[g]), part[9 + 2 * g])
+        for g in range(len(table_shapes))
     ]
     return StepContext(
-        n_tokens=T, n_seqs=B, act_dtype=act_dtype, tokens=part[0], positions=part[1], seq_of_token=part[2],
-        q_start=part[3], kv_len=part[4], slot_ids=part[5], out_rows=part[6], groups=groups, q_lens=q_lens,
-        n_cached=n_cached, slot_ids_host=slot_ids, n_out=len(out_rows),
+        n_tokens=int(host["q_start"][-1]), n_seqs=len(host["q_lens"]), act_dtype=act_dtype,
+        seq_records=part[0].view(-1, 4), tokens=part[1],
+        positions=part[2], seq_of_token=part[3], q_start=part[4], kv_len=part[5], slot_ids=part[6],
+        out_rows=part[7], groups=groups, q_lens=host["q_lens"], n_cached=host["n_cached"],
+        slot_ids_host=host["slot_ids"], q_start_host=host["q_start"], n_out=host["n_out"],
     )
+
+
+def build_context(entries: Sequence[StepEntry], cache: CacheManager, act_dtype: torch.dtype,
+                  device: torch.device | str, vocab_size: Optional[int] = None) -> StepContext:
+    """Host vectors for ``entries`` (whose pages are already reserved), packed
+    into one int32 buffer and copied to the device once."""
+    packed, offs, table_shapes, host = pack_context(entries, cache, vocab_size)
+    return context_from_packed(torch.from_numpy(packed).to(device), offs, table_shapes, host, cache.page_size,
+                               act_dtype)

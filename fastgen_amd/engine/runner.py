@@ -10,14 +10,62 @@ is one, because a decoded token is a portion of length one.
 
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Optional, Sequence
+import os
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage, group_entries
-from .context import StepContext, StepEntry, build_context
+from .context import StepContext, StepEntry, build_context, context_from_packed, pack_context
 from .model import Model
+
+
+class _DecodeGraph:
+    """One captured decode step for a fixed number of sequences.
+
+    The step's int32 vectors live in a device buffer of fixed layout (block
+    tables as wide as a request can get); a replay copies the new values in
+    and runs the captured kernels, which read lengths and pages from that
+    buffer.  (The reference captures 16 such graphs at spaced batch sizes and
+    pads, ``fastgen/generate.py:296-352``; here a graph is captured for each
+    batch size when it first occurs.)
+    """
+
+    def __init__(self, runner: "ModelRunner", entries: Sequence[StepEntry]) -> None:
+        model, cache = runner.model, runner.cache
+        packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, runner.table_width)
+        self.layout = (tuple(int(o) for o in offs), tuple(shapes))
+        self.staging = torch.empty(packed.size, dtype=torch.int32, pin_memory=True)
+        self.staging.numpy()[:] = packed
+        self.packed = self.staging.to(model.device)
+        self.copied = torch.cuda.Event()
+        self.ctx = context_from_packed(self.packed, offs, shapes, host, cache.page_size, model.dtype)
+        self.ctx.graph_capacity = runner.table_width * cache.page_size
+        # warm up outside the capture (libraries load, the matrix library picks its kernels), then capture
+        side = torch.cuda.Stream(device=model.device)
+        side.wait_stream(torch.cuda.current_stream(model.device))
+        with torch.cuda.stream(side):
+            model.forward(self.ctx, runner.stores)
+        torch.cuda.current_stream(model.device).wait_stream(side)
+        torch.cuda.synchronize(model.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=runner.graph_pool):
+            self.logits = model.forward(self.ctx, runner.stores)
+        runner.graph_pool = runner.graph_pool or self.graph.pool()
+
+    def replay(self, runner: "ModelRunner", entries: Sequence[StepEntry]) -> torch.Tensor:
+        packed, offs, shapes, host = pack_context(entries, runner.cache, runner.model.vocab_size,
+                                                  runner.table_width)
+        if (tuple(int(o) for o in offs), tuple(shapes)) != self.layout:
+            raise RuntimeError("decode graph: the step's layout differs from the captured one")
+        self.copied.synchronize()  # the staging buffer is free again
+        self.staging.numpy()[:] = packed
+        self.packed.copy_(self.staging, non_blocking=True)
+        self.copied.record()
+        self.graph.replay()
+        return self.logits
 
 
 class ModelRunner:
@@ -42,6 +90,14 @@ class ModelRunner:
             self.storage.store_for(i, e.reads_cache_of) for i, e in enumerate(model.layout.order)
         ]
         self.last_context: Optional[StepContext] = None
+        # decode graphs: FG_NO_GRAPHS=1 switches them off (the reference: FG_NO_CUDA_GRAPHS)
+        # a mixer with state of its own is stepped eagerly: the warm-up run before a capture would
+        # advance its state twice
+        self.use_graphs = os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and not model.state_needs()
+        self.table_width = max(1, max(pages, default=1))
+        self.graphs: Dict[int, _DecodeGraph] = {}
+        self.graph_pool = None
+        self.max_graphs = 32
 
     # ------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> int:
@@ -72,9 +128,30 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """fp32 logits ``[n_wanted, vocab]`` in the order of the entries and
         of their ``want`` lists; None if nothing is wanted."""
-        ctx = self.prepare(entries)
-        self.last_context = ctx
-        logits = self.model.forward(ctx, self.stores)
+        if self.use_graphs and self._is_plain_decode(entries):
+            logits = self._graph_step(entries)
+        else:
+            ctx = self.prepare(entries)
+            self.last_context = ctx
+            logits = self.model.forward(ctx, self.stores)
         for e in entries:
             self.cache.advance(e.rid, len(e.tokens))
         return logits
+
+    # ------------------------------------------------------- decode graphs
+    def _is_plain_decode(self, entries: Sequence[StepEntry]) -> bool:
+        """One token a request, its logits wanted, every request already live."""
+        return bool(entries) and all(
+            len(e.tokens) == 1 and list(e.want) == [0] and self.cache.is_live(e.rid) for e in entries
+        ) and (len(entries) in self.graphs or len(self.graphs) < self.max_graphs)
+
+    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        if len({e.rid for e in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
+        for e in entries:
+            self.cache.reserve(e.rid, 1)
+        g = self.graphs.get(len(entries))
+        if g is None:
+            g = self.graphs[len(entries)] = _DecodeGraph(self, entries)
+            # the capture ran the step's kernels only as a recording: replay it for this step's result
+        return g.replay(self, entries)

@@ -33,7 +33,7 @@ HIPCC_FLAGS = [
     # packed fp32 instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "kv_layout.h"]
 
 # library name -> source file
 LIBRARIES: Dict[str, str] = {
@@ -42,6 +42,11 @@ LIBRARIES: Dict[str, str] = {
     "attention": "attention.hip",
     "gemm": "gemm.hip",
     "sampling": "sampling.hip",
+}
+
+# libraries compiled once per value of a macro: name -> (source, macro, values that build_all compiles)
+VARIANT_LIBRARIES: Dict[str, tuple] = {
+    "attention_mfma": ("attention_mfma.hip", "FG_HD", tuple(range(16, 257, 16))),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -66,12 +71,22 @@ def _hipcc() -> str:
     )
 
 
+def _split_variant(name: str):
+    """``attention_mfma@128`` -> (source file, ["-DFG_HD=128"], file stem)."""
+    if "@" in name:
+        base, value = name.split("@", 1)
+        src, macro, _ = VARIANT_LIBRARIES[base]
+        return src, [f"-D{macro}={int(value)}"], f"{base}_{int(value)}"
+    return LIBRARIES[name], [], name
+
+
 def _source_hash(name: str) -> str:
+    src, defines, _ = _split_variant(name)
     h = hashlib.sha256()
-    for f in [LIBRARIES[name], *HEADERS]:
+    for f in [src, *HEADERS]:
         h.update(f.encode())
         h.update((CSRC / f).read_bytes())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + defines).encode())
     return h.hexdigest()[:12]
 
 
@@ -82,7 +97,7 @@ def _build_dirs() -> Iterable[Path]:
 
 
 def _lib_filename(name: str) -> str:
-    return f"libfg_{name}-{_source_hash(name)}.so"
+    return f"libfg_{_split_variant(name)[2]}-{_source_hash(name)}.so"
 
 
 def find_built(name: str) -> Optional[Path]:
@@ -109,13 +124,14 @@ def _writable_dir() -> Path:
 
 def compile_library(name: str, *, verbose: bool = True) -> Path:
     """Compile one library now (also when a built one exists) and return its path."""
-    src = CSRC / LIBRARIES[name]
+    src_name, defines, stem = _split_variant(name)
+    src = CSRC / src_name
     out_dir = _writable_dir()
     out = out_dir / _lib_filename(name)
     tmp_out = out_dir / f".{out.name}.{os.getpid()}-{threading.get_ident()}.tmp"
-    cmd = [_hipcc(), *HIPCC_FLAGS, f"-I{CSRC}", str(src), "-o", str(tmp_out)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *defines, f"-I{CSRC}", str(src), "-o", str(tmp_out)]
     if verbose:
-        print(f"[fastgen_amd] compiling {src.name} for {ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[fastgen_amd] compiling {src.name} {' '.join(defines)} for {ARCH} ...", file=sys.stderr, flush=True)
     t0 = time.time()
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # a long compile says so now and then
@@ -139,7 +155,7 @@ def compile_library(name: str, *, verbose: bool = True) -> Path:
         raise KernelBuildError(f"hipcc failed for {src}:\n{' '.join(cmd)}\n{log}")
     os.replace(tmp_out, out)
     # libraries of older sources are of no use any more
-    for old in out_dir.glob(f"libfg_{name}-*.so"):
+    for old in out_dir.glob(f"libfg_{stem}-*.so"):
         if old != out:
             old.unlink(missing_ok=True)
     if verbose:
@@ -149,12 +165,13 @@ def compile_library(name: str, *, verbose: bool = True) -> Path:
     return out
 
 
-def build_all(*, force: bool = True, verbose: bool = True, jobs: int = 4) -> Dict[str, Path]:
+def build_all(*, force: bool = True, verbose: bool = True, jobs: int = 8) -> Dict[str, Path]:
     """Compile every kernel library (``force``: also those already built)."""
     from concurrent.futures import ThreadPoolExecutor
 
-    names = [n for n in LIBRARIES if force or find_built(n) is None]
-    out = {n: find_built(n) for n in LIBRARIES if n not in names}
+    every = list(LIBRARIES) + [f"{b}@{v}" for b, (_, _, values) in VARIANT_LIBRARIES.items() for v in values]
+    names = [n for n in every if force or find_built(n) is None]
+    out = {n: find_built(n) for n in every if n not in names}
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
         for n, p in zip(names, ex.map(lambda n: compile_library(n, verbose=verbose), names)):
             out[n] = p
@@ -170,7 +187,7 @@ def load(name: str) -> ctypes.CDLL:
         lib = _loaded.get(name)
         if lib is not None:
             return lib
-        if name not in LIBRARIES:
+        if name not in LIBRARIES and name.split("@")[0] not in VARIANT_LIBRARIES:
             raise KeyError(f"no kernel library named {name!r}")
         path = find_built(name) or compile_library(name)
         try:

@@ -205,15 +205,120 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
     return out
 
 
+MFMA_MAX_HEAD_DIM = 256
+_SPLIT_TARGET_BLOCKS = 1024  # workgroups wanted in flight for the decode kernel (4 per CU)
+
+
+def attention_items(q_lens, q_start, n_cached, group_size: int):
+    """Cut the step's sequences into items for the MFMA kernels.
+
+    Returns two int32 arrays ``[n, 4]`` of (sequence, first flat token, tokens,
+    position of the first token): items of at most 16 rows for the split
+    kernel (decoded tokens and very short portions) and items of at most 64
+    rows for the tile kernel.
+    """
+    import numpy as np
+
+    small, big = [], []
+    per_tile = max(1, 64 // group_size)
+    for b, n in enumerate(q_lens):
+        n, s, c = int(n), int(q_start[b]), int(n_cached[b])
+        if n * group_size <= 16:
+            small.append((b, s, n, c))
+        else:
+            big.extend((b, s + i, min(per_tile, n - i), c + i) for i in range(0, n, per_tile))
+    as_arr = lambda x: np.asarray(x, dtype=np.int32).reshape(-1, 4)
+    return as_arr(small), as_arr(big)
+
+
+def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                         block_table: torch.Tensor, small_items: Optional[torch.Tensor],
+                         big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
+                         n_splits: int = 1) -> torch.Tensor:
+    """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
+    device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
+    every query token of the step must be covered by exactly one item."""
+    _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items)
+    n_pages, n_kv, page_size, hd = k_pages.shape
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
+          and v_pages.dtype == torch.bfloat16, "the MFMA attention kernels take bfloat16")
+    _need(hd % 16 == 0 and hd <= MFMA_MAX_HEAD_DIM, f"head size {hd}: multiples of 16 up to {MFMA_MAX_HEAD_DIM}")
+    _need(k_pages.is_contiguous() and v_pages.is_contiguous() and v_pages.shape == (n_pages, n_kv, hd, page_size),
+          "k_pages [n_pages, KV, P, hd] and v_pages [n_pages, KV, hd, P] must be contiguous")
+    _need(n_heads % n_kv == 0 and page_size % 8 == 0, "heads must be a multiple of kv heads, pages of 8 tokens")
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * hd and q.stride(0) % 8 == 0
+          and q.data_ptr() % 16 == 0, "q must be [T, >= H*hd], rows 16-byte aligned")
+    _need(out.shape == (T, n_heads * hd) and out.stride(1) == 1 and out.stride(0) % 4 == 0, "out must be [T, H*hd]")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, max_pages]")
+    lib = _lib.load(f"attention_mfma@{hd}")
+    G = n_heads // n_kv
+    if small_items is not None and small_items.numel():
+        _need(G <= 16, "the split kernel takes at most 16 query heads per kv head")
+        _i32(small_items, "small_items")
+        _need(small_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
+        n = small_items.numel() // 4
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty((n * n_kv * n_splits * 16, hd), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((n * n_kv * n_splits * 16, 2), dtype=torch.float32, device=q.device)
+        for i0 in range(0, n, 65535):  # grid.z limit
+            ni = min(65535, n - i0)
+            st = lib.fg_attn_split(
+                _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                block_table.stride(0), ctypes.c_void_p(small_items.data_ptr() + 16 * i0), ni,
+                ctypes.c_void_p(part_o.data_ptr() + 4 * i0 * n_kv * n_splits * 16 * hd if part_o is not None else 0),
+                ctypes.c_void_p(part_ml.data_ptr() + 4 * i0 * n_kv * n_splits * 16 * 2 if part_ml is not None else 0),
+                n_splits, n_heads, n_kv, hd, page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
+            _check(st, "attn_split")
+    if big_items is not None and big_items.numel():
+        _need(G <= 64, "the tile kernel takes at most 64 query heads per kv head")
+        _i32(big_items, "big_items")
+        _need(big_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
+        st = lib.fg_attn_tile(
+            _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            block_table.stride(0), _ptr(big_items), big_items.numel() // 4, n_heads, n_kv, hd, page_size,
+            ctypes.c_float(scale), int(window or 0), _stream(q))
+        _check(st, "attn_tile")
+    return out
+
+
 def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                     group, ctx, n_heads: int, scale: float, window: int = 0) -> torch.Tensor:
-    """Attention for one step: picks the kernel for the step's shape.
+    """Attention for one step: picks the kernel for the step's dtype and shape.
 
     ``group`` carries the block table of the layer's cache group, ``ctx`` the
-    step's per-token vectors (``fastgen_amd.engine.context``).
+    step's per-token vectors (``fastgen_amd.engine.context``).  bfloat16 with a
+    head size in steps of 16 up to 256 and at most 16 query heads per kv head
+    runs on the matrix cores; everything else (float32 always) runs the general
+    kernel.
     """
-    return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token,
-                                   ctx.positions, n_heads, scale, window)
+    n_kv, hd = k_pages.shape[1], k_pages.shape[3]
+    G = n_heads // n_kv
+    if q.dtype != torch.bfloat16 or hd % 16 or hd > MFMA_MAX_HEAD_DIM or G > 16:
+        return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token,
+                                       ctx.positions, n_heads, scale, window)
+    plan = ctx.scratch.get(("attention_items", G))
+    if plan is None:
+        import numpy as np
+
+        if ctx.seq_records is not None and int(ctx.q_lens.max()) * G <= 16:
+            # every sequence is one item of the split kernel: its records are in the step's buffer
+            # already (and are refreshed with it when the step is a replayed graph)
+            plan = (ctx.seq_records, None, ctx.n_seqs)
+        else:
+            small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G)
+            both = torch.from_numpy(np.concatenate([small, big]).reshape(-1)).to(q.device)
+            plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small))
+        ctx.scratch[("attention_items", G)] = plan
+    small_d, big_d, n_small = plan
+    n_splits = 1
+    if n_small:
+        tiles = -(-(ctx.graph_capacity or ctx.max_kv_len) // 64)
+        n_splits = max(1, min(-(-tiles // 4), -(-_SPLIT_TARGET_BLOCKS // (n_small * n_kv)), 64))
+    return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
+                                window, n_splits)
 
 
 # ----------------------------------------------------------------------- gemm

@@ -15,6 +15,8 @@ from plain_llama import (
     plain_top_p_keep,
 )
 
+from fastgen_amd.cache.layout import pack_k, pack_v, unpack_k, unpack_v
+
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
@@ -123,16 +125,17 @@ def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P):
     got = qkv_d.cpu()
     assert torch.allclose(got[:, : H * hd].float(), rotate(q).reshape(T, -1).float(), **tol(dtype))
     assert torch.equal(got[:, (H + KV) * hd :], qkv[:, (H + KV) * hd :])  # v untouched in place
-    want_k, want_v = kp.clone(), vp.clone()
+    want_k, want_v = torch.full((n_pages, KV, P, hd), 7.0, dtype=dtype), torch.full((n_pages, KV, P, hd), 7.0, dtype=dtype)
     rk = rotate(k)
     for t in range(T):
         s = int(slots[t])
         if s < 0:
             continue
         want_k[s // P, :, s % P, :] = rk[t]
-        want_v[s // P, :, :, s % P] = v[t]
-    assert torch.allclose(kp_d.cpu().float(), want_k.float(), **tol(dtype))
-    assert torch.equal(vp_d.cpu(), want_v)  # nothing else in the pool changed either
+        want_v[s // P, :, s % P, :] = v[t]
+    # the pool in natural order: key p of a page at [p, :], whatever the storage order inside the page
+    assert torch.allclose(unpack_k(kp_d.cpu()).float(), want_k.float(), **tol(dtype))
+    assert torch.equal(unpack_v(vp_d.cpu()), want_v)  # nothing else in the pool changed either
 
 
 # ---------------------------------------------------------------- attention
@@ -162,9 +165,13 @@ def _paged_case(dtype, seqs, H, KV, hd, P, seed, poison=True, peak=None):
             q[qpos, qh, 0] = 12.0 * math.sqrt(hd)
         pages = [perm.pop() for _ in range(pages_of[b])]
         table[b, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
-        for p in range(n):
-            kp[pages[p // P], :, p % P, :] = k[p]
-            vp[pages[p // P], :, :, p % P] = v[p]
+        for j, pg in enumerate(pages):  # natural [KV, P, hd] per page, then into storage order
+            nk = torch.full((KV, P, hd), fill, dtype=dtype)
+            nv = torch.full((KV, P, hd), fill, dtype=dtype)
+            cnt = min(P, n - j * P)
+            nk[:, :cnt] = k[j * P : j * P + cnt].transpose(0, 1)
+            nv[:, :cnt] = v[j * P : j * P + cnt].transpose(0, 1)
+            kp[pg], vp[pg] = pack_k(nk), pack_v(nv)
         qs.append(q), ks.append(k), vs.append(v)
         q_rows.append(q[n0:].reshape(n1, H * hd))
         seq_of += [b] * n1
@@ -344,3 +351,81 @@ def test_kernels_refuse_what_they_cannot_take(ops):
         ops.paged_attention_general(q, torch.empty_like(q), kp, vp, i.view(1, 1), i, i, 2, 1.0)
     with pytest.raises(KernelArgumentError, match="GPU only"):
         ops.silu_mul(torch.zeros(2, 4))
+
+
+# ------------------------------------------------------- attention on MFMA
+def _run_mfma(ops, case, seqs, H, KV, window=0, n_splits=1):
+    import numpy as np
+
+    q_lens = [b for _, b in seqs]
+    q_start = np.concatenate([[0], np.cumsum(q_lens)])
+    small, big = ops.attention_items(q_lens, q_start, [a for a, _ in seqs], H // KV)
+    dev = lambda a: torch.from_numpy(a.reshape(-1)).to(DEV) if a.size else None
+    out = torch.full_like(case["q"], float("nan"))
+    ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], dev(small), dev(big), H,
+                             case["kp"].shape[3] ** -0.5, window, n_splits)
+    return out, len(small), len(big)
+
+
+MFMA_SHAPES = [
+    # H, KV, hd, P
+    (4, 2, 16, 16),
+    (5, 1, 48, 32),
+    (6, 3, 32, 8),
+    (32, 8, 128, 64),
+    (3, 3, 80, 128),
+    (16, 1, 64, 16),
+    (2, 1, 256, 32),
+    (7, 7, 112, 24),
+]
+MFMA_SEQS = [(0, 1), (0, 70), (131, 1), (60, 9), (17, 2), (255, 1), (0, 129), (300, 3), (63, 66)]
+
+
+@pytest.mark.parametrize("H,KV,hd,P", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 37, 150])
+@pytest.mark.parametrize("n_splits", [1, 3])
+def test_paged_attention_mfma(ops, H, KV, hd, P, window, n_splits):
+    case = _paged_case(torch.bfloat16, MFMA_SEQS, H, KV, hd, P, seed=21)
+    out, n_small, n_big = _run_mfma(ops, case, MFMA_SEQS, H, KV, window, n_splits)
+    assert n_small and n_big  # both kernels run
+    want = _plain_rows(case, MFMA_SEQS, window or None)
+    assert torch.isfinite(out).all()  # every row written, no poison read
+    assert torch.allclose(out.cpu().float(), want, atol=1.5e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 8])
+def test_paged_attention_mfma_far_key_and_edges(ops, n_splits):
+    """A key that gets nearly all the weight, at the edges of tiles, pages and
+    splits, for a decoded token (split kernel) and inside a portion (tile
+    kernel)."""
+    H, KV, hd, P = 8, 2, 64, 16
+    for kpos in (0, 15, 16, 63, 64, 127, 128, 300, 399, 400):
+        for seqs, qpos, row in (([(0, 3), (400, 1), (10, 2)], 400, 3), ([(0, 2), (380, 40)], 400, 2 + 20)):
+            case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=22, peak=(1, qpos, 5, kpos))
+            out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, n_splits)
+            v = case["whole"][2][1]
+            got = out.cpu().float()[row].view(H, hd)[5]
+            assert torch.allclose(got, v[kpos, 1].float(), atol=2e-2), (kpos, seqs)
+            assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
+
+
+def test_paged_attention_mfma_window_edge(ops):
+    H, KV, hd, P, w = 4, 1, 32, 16, 40
+    for seqs, row in (([(100, 1)], 0), ([(90, 30)], 10)):
+        for kpos, seen in ((100 - w, False), (100 - w + 1, True)):
+            case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=23, peak=(0, 100, 1, kpos))
+            out, _, _ = _run_mfma(ops, case, seqs, H, KV, w, 2)
+            v = case["whole"][2][0]
+            got = out.cpu().float()[row].view(H, hd)[1]
+            assert torch.allclose(got, v[kpos, 0].float(), atol=2e-2) == seen
+            assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs, w), atol=1.5e-2, rtol=2e-2)
+
+
+def test_paged_attention_mfma_long_context(ops):
+    """Llama-3.1-8B's attention shape at a context of several thousand keys,
+    one decoded token and one long portion."""
+    H, KV, hd, P = 32, 8, 128, 64
+    seqs = [(5000, 1), (3000, 200)]
+    case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=24, poison=True)
+    out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, 16)
+    assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
