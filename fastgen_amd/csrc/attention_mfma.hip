@@ -38,6 +38,23 @@ constexpr int TILE = 64;             // keys per tile
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Bit masks that zero the value slots of keys outside [lo, hi]; slot e of a
+// chunk is key ka + (e & 3) + 16 * (e >> 2).  Branch-free, so that it can sit
+// between loads without splitting them up.
+__device__ __forceinline__ u32x4 slot_mask(int ka, int lo, int hi) {
+  u32x4 m;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int k_even = ka + ((2 * w) & 3) + 16 * ((2 * w) >> 2), k_odd = k_even + 1;
+    m[w] = ((k_even >= lo && k_even <= hi) ? 0x0000ffffu : 0u) | ((k_odd >= lo && k_odd <= hi) ? 0xffff0000u : 0u);
+  }
+  return m;
+}
+__device__ __forceinline__ bf16x8 and_mask(bf16x8 v, u32x4 m) {
+  return __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, v) & m);
+}
 
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
@@ -83,14 +100,27 @@ template <class LK, class LV>
 __device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf16x8 (&qop)[NKS], float scale,
                                             float& m, float& l, f32x4 (&o)[NDB], LK load_k, LV load_v) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
+  // The order of the loads in the source is the order in which they are issued: all of K, then the
+  // first half of V, are in flight before the first MFMA waits for anything; the second half of V is
+  // issued when K's registers are free and flies during the softmax.
+  bf16x8 kop[4][NKS];
+#pragma unroll
+  for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) kop[kb][ks] = load_k(kb, ks);
+  bf16x8 vop0[NDB], vop1[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) vop0[db] = load_v(db, 0);
   f32x4 s[4];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
     s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
-      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_k(kb, ks), qop[ks], s[kb], 0, 0, 0);
+      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[kb][ks], qop[ks], s[kb], 0, 0, 0);
   }
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) vop1[db] = load_v(db, 1);
   float mx = -INFINITY;
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb)
@@ -121,19 +151,21 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf
 #pragma unroll
   for (int db = 0; db < NDB; ++db) {
     o[db] *= alpha;
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load_v(db, ks), pop[ks], o[db], 0, 0, 0);
+    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0[db], pop[0], o[db], 0, 0, 0);
   }
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1[db], pop[1], o[db], 0, 0, 0);
 }
 
-// Q^T operand: lane holds Q[row lane%16][32*ks + 8*(lane/16) ..+7]
-__device__ __forceinline__ void load_q(bf16x8 (&qop)[NKS], const bf16_t* qrow /* null: padding row */) {
+// qrow is always a readable row; `valid` says whether it is this lane's
+__device__ __forceinline__ void load_q(bf16x8 (&qop)[NKS], const bf16_t* qrow, bool valid) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
     const int d = 32 * ks + 8 * g;
-    qop[ks] = (qrow && d < HD) ? *(const bf16x8*)(qrow + d) : zero8();
+    const bf16x8 v = *(const bf16x8*)(qrow + (d < HD ? d : 0));  // loads are never conditional
+    qop[ks] = (valid && d < HD) ? v : zero8();
   }
 }
 
@@ -141,6 +173,7 @@ __device__ __forceinline__ void load_q(bf16x8 (&qop)[NKS], const bf16_t* qrow /*
 // grid (n_splits, n_kv, n_items), 256 threads.  items: [n_items][4] = sequence,
 // flat index of the first token, number of tokens, position of the first
 // token; n_tok * (H / KV) <= 16.
+template <bool PERM /* the page's value slots are permuted: page_size % 32 == 0 */>
 __global__ __launch_bounds__(256) void attn_split_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
@@ -160,14 +193,14 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   const int pos_last = it.pos0 + it.n_tok - 1;
   const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
   ItemRows me{-1, 0};
-  const bf16_t* qrow = nullptr;
-  if (r16 < it.n_tok * G) {
-    me.pos = it.pos0 + r16 / G;
+  const bool my_row = r16 < it.n_tok * G;
+  const int my_tok = my_row ? r16 / G : 0, my_head = my_row ? r16 % G : 0;
+  if (my_row) {
+    me.pos = it.pos0 + my_tok;
     me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
-    qrow = q + (size_t)(it.tok0 + r16 / G) * q_stride + (size_t)(kvh * G + r16 % G) * HD;
   }
   bf16x8 qop[NKS];
-  load_q(qop, qrow);
+  load_q(qop, q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
 
   const int t_lo = first_min / TILE, t_hi = pos_last / TILE;
   const int per_split = (t_hi - t_lo + 1 + n_splits - 1) / n_splits;
@@ -182,63 +215,55 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   const size_t head_elems = (size_t)page_size * HD;  // elements of one kv head in a page
   for (int t = t_begin + wave; t < t_end; t += 4) {
     const int k0 = t * TILE;
+    // Loads are never conditional (a branch around a load keeps the compiler from issuing the
+    // tile's loads together): addresses are clamped into the item's key range and what lies
+    // outside is masked afterwards.
     // K chunks of this lane: key 16*kb + r16 of the tile, head dims 32*ks + 8*g
     const bf16_t* kptr[4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
-      const int key = k0 + 16 * kb + r16;
-      kptr[kb] = nullptr;
-      if (key >= first_min && key <= pos_last)
-        kptr[kb] = k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
-                   lay.k_off(pager.in_page(key), 8 * g);
+      const int key = min(max(k0 + 16 * kb + r16, first_min), pos_last);  // masked by the scores' select
+      kptr[kb] = k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                 lay.k_off(pager.in_page(key), 8 * g);
     }
     // V chunks of this lane: keys 32*ks + 4*g + (0..3) and 16 more on; head dim 16*db + r16
     const bf16_t* vptr[2][2];
-    bool vedge[2];
+    u32x4 vmask[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const int ka = k0 + 32 * ks + 4 * g, kb2 = ka + 16;
-      vedge[ks] = ka < first_min || kb2 + 3 > pos_last;
-      vptr[ks][0] = vptr[ks][1] = nullptr;
-      if (ka + 3 >= first_min && ka <= pos_last)
-        vptr[ks][0] = v_pages + ((size_t)pager.page_of(ka) * n_kv + kvh) * head_elems +
-                      lay.v_off(pager.in_page(ka), r16);
-      if (!lay.permuted && kb2 + 3 >= first_min && kb2 <= pos_last)
-        vptr[ks][1] = v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
-                      lay.v_off(pager.in_page(kb2), r16);
-      if (lay.permuted && !vptr[ks][0] && kb2 + 3 >= first_min && kb2 <= pos_last)
-        // the first half lies outside the range but the second inside: same chunk, same page
-        vptr[ks][0] = v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
-                      lay.v_off(pager.in_page(kb2), r16) - 4;
+      vmask[ks] = slot_mask(ka, first_min, pos_last);  // what lies outside may hold anything, NaN included
+      const bool in_a = ka + 3 >= first_min && ka <= pos_last;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        // a key of the wanted run if it has one in range, else any key in range
+        const int want = (half == 0 && (in_a || !PERM)) ? ka : kb2;
+        const int x = min(max(want, first_min), pos_last);
+        const int xin = pager.in_page(x);
+        const int back = PERM ? (lay.v_slot(xin) & 7) : (xin & 3);  // to the start of the chunk / run of 4
+        vptr[ks][half] = v_pages + ((size_t)pager.page_of(x) * n_kv + kvh) * head_elems + lay.v_off(xin, r16) - back;
+      }
     }
-    const size_t k_step = (size_t)4 * lay.kb * 8;       // 32 head dims on: 4 chunks of kb keys
-    const size_t v_step = (size_t)(page_size / 8) * 128;  // 16 head dims on: one dim block
+    const size_t k_step = lay.k_step32(), v_step = lay.v_step_block();
     auto load_k = [&](int kb, int ks) -> bf16x8 {
-      return (kptr[kb] && 32 * ks + 8 * g < HD) ? *(const bf16x8*)(kptr[kb] + ks * k_step) : zero8();
+      const bool in = 32 * ks + 8 * g < HD;
+      const bf16x8 v = *(const bf16x8*)(kptr[kb] + (in ? ks * k_step : 0));
+      return in ? v : zero8();
     };
     auto load_v = [&](int db, int ks) -> bf16x8 {
-      bf16x8 v = zero8();
-      if (lay.permuted) {
-        if (vptr[ks][0]) v = *(const bf16x8*)(vptr[ks][0] + db * v_step);
+      bf16x8 v;
+      if (PERM) {
+        v = *(const bf16x8*)(vptr[ks][0] + db * v_step);
       } else {
-        bf16x4 lo = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f}, hi = lo;
-        if (vptr[ks][0]) lo = *(const bf16x4*)(vptr[ks][0] + db * v_step);
-        if (vptr[ks][1]) hi = *(const bf16x4*)(vptr[ks][1] + db * v_step);
+        const bf16x4 lo = *(const bf16x4*)(vptr[ks][0] + db * v_step);
+        const bf16x4 hi = *(const bf16x4*)(vptr[ks][1] + db * v_step);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           v[e] = lo[e];
           v[4 + e] = hi[e];
         }
       }
-      if (vedge[ks]) {  // keys outside the item's range may hold anything, NaN included
-        const int ka = k0 + 32 * ks + 4 * g;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int kk = ka + (e & 3) + 16 * (e >> 2);
-          if (kk < first_min || kk > pos_last) v[e] = (__bf16)0.f;
-        }
-      }
-      return v;
+      return and_mask(v, vmask[ks]);
     };
     attend_tile(k0, me, qop, scale, m, l, o, load_k, load_v);
   }
@@ -339,10 +364,13 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
       n_splits < 1 || n_splits > 65535 || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
       out_stride % 4 || (n_splits > 1 && (!part_o || !part_ml)))
     return FG_ERR_ARG;
-  attn_split_kernel<<<dim3(n_splits, n_kv, n_items), 256, 0, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-      block_table, bt_stride, items, part_o, part_ml, n_heads, n_kv, page_size, page_shift_of(page_size), scale,
-      window);
+#define LAUNCH(PERM)                                                                                           \
+  attn_split_kernel<PERM><<<dim3(n_splits, n_kv, n_items), 256, 0, stream>>>(                                  \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,    \
+      block_table, bt_stride, items, part_o, part_ml, n_heads, n_kv, page_size, page_shift_of(page_size), scale, \
+      window)
+  if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
+#undef LAUNCH
   if (n_splits > 1)
     attn_combine_kernel<<<dim3(16, n_kv, n_items), HD < 64 ? 64 : HD, 0, stream>>>(
         part_o, part_ml, items, (bf16_t*)out, out_stride, n_heads, n_kv, n_splits);
@@ -354,6 +382,7 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
 // 64 / (H / KV) tokens.  The K and V tiles go through LDS in the order the
 // operands are read: K [4 key blocks][HD/8 chunks][16 keys][8], V [HD/16 dim
 // blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
+template <bool PERM>
 __global__ __launch_bounds__(256) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
@@ -373,14 +402,14 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
 
   const int row = wave * 16 + r16;
   ItemRows me{-1, 0};
-  const bf16_t* qrow = nullptr;
-  if (row < it.n_tok * G) {
-    me.pos = it.pos0 + row / G;
+  const bool my_row = row < it.n_tok * G;
+  const int my_tok = my_row ? row / G : 0, my_head = my_row ? row % G : 0;
+  if (my_row) {
+    me.pos = it.pos0 + my_tok;
     me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
-    qrow = q + (size_t)(it.tok0 + row / G) * q_stride + (size_t)(kvh * G + row % G) * HD;
   }
   bf16x8 qop[NKS];
-  load_q(qop, qrow);
+  load_q(qop, q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
   // the keys this wave's rows can see: tiles outside are skipped by the wave
   int w_hi = me.pos, w_lo = me.pos < 0 ? 0x7fffffff : me.first;
 #pragma unroll
@@ -398,49 +427,43 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   constexpr int KCH = HD / 8;  // 16-byte chunks in a key
   for (int k0 = (first_min / TILE) * TILE; k0 <= pos_last; k0 += TILE) {
     __syncthreads();  // the previous tile is no longer read
+    // (loads are never conditional: addresses are clamped into the item's key range, what lies
+    // outside is masked; keys beyond the range give scores that the select discards)
     // K: chunk (block kb, dims 8c.., key r) -> k_s[((kb*KCH + c)*16 + r)*8]; r fastest over threads
     for (int w = threadIdx.x; w < TILE * KCH; w += 256) {
-      const int r = w & 15, c = (w >> 4) % KCH, kb = (w >> 4) / KCH, key = k0 + 16 * kb + r;
-      bf16x8 v = zero8();
-      if (key >= first_min && key <= pos_last)
-        v = *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
-                             lay.k_off(pager.in_page(key), 8 * c));
-      *(bf16x8*)(k_s + (size_t)w * 8) = v;
+      const int r = w & 15, c = (w >> 4) % KCH, kb = (w >> 4) / KCH;
+      const int key = min(max(k0 + 16 * kb + r, first_min), pos_last);
+      *(bf16x8*)(k_s + (size_t)w * 8) =
+          *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                           lay.k_off(pager.in_page(key), 8 * c));
     }
     // V: chunk (dim block db, key chunk kc = 4*ks + gg, dim r) -> v_s[((db*8 + kc)*16 + r)*8];
     // its slots are keys 32*ks + 4*gg + (0..3) and 16 more on
     for (int w = threadIdx.x; w < NDB * 8 * 16; w += 256) {
       const int r = w & 15, kc = (w >> 4) & 7, db = w >> 7;
       const int ka = k0 + 32 * (kc >> 2) + 4 * (kc & 3), kb2 = ka + 16;
-      bf16x8 v = zero8();
-      const bool in_a = ka + 3 >= first_min && ka <= pos_last, in_b = kb2 + 3 >= first_min && kb2 <= pos_last;
-      if (lay.permuted) {
-        if (in_a || in_b) {
-          const int kk = in_a ? ka : kb2;
-          v = *(const bf16x8*)(v_pages + ((size_t)pager.page_of(kk) * n_kv + kvh) * head_elems +
-                               lay.v_off(pager.in_page(kk), 16 * db + r) - (in_a ? 0 : 4));
-        }
+      const bool in_a = ka + 3 >= first_min && ka <= pos_last;
+      const bf16_t* src[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int want = (half == 0 && (in_a || !PERM)) ? ka : kb2;
+        const int x = min(max(want, first_min), pos_last);
+        const int xin = pager.in_page(x);
+        const int back = PERM ? (lay.v_slot(xin) & 7) : (xin & 3);
+        src[half] = v_pages + ((size_t)pager.page_of(x) * n_kv + kvh) * head_elems + lay.v_off(xin, 16 * db + r) - back;
+      }
+      bf16x8 v;
+      if (PERM) {
+        v = *(const bf16x8*)src[0];
       } else {
-        bf16x4 lo = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f}, hi = lo;
-        if (in_a)
-          lo = *(const bf16x4*)(v_pages + ((size_t)pager.page_of(ka) * n_kv + kvh) * head_elems +
-                                lay.v_off(pager.in_page(ka), 16 * db + r));
-        if (in_b)
-          hi = *(const bf16x4*)(v_pages + ((size_t)pager.page_of(kb2) * n_kv + kvh) * head_elems +
-                                lay.v_off(pager.in_page(kb2), 16 * db + r));
+        const bf16x4 lo = *(const bf16x4*)src[0], hi = *(const bf16x4*)src[1];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           v[e] = lo[e];
           v[4 + e] = hi[e];
         }
       }
-      if (ka < first_min || kb2 + 3 > pos_last) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int kk = ka + (e & 3) + 16 * (e >> 2);
-          if (kk < first_min || kk > pos_last) v[e] = (__bf16)0.f;
-        }
-      }
+      v = and_mask(v, slot_mask(ka, first_min, pos_last));
       *(bf16x8*)(v_s + (size_t)w * 8) = v;
     }
     __syncthreads();
@@ -477,9 +500,12 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 64 || page_size < 8 || page_size % 8 ||
       n_kv > 65535 || window < 0 || q_stride % 8 || out_stride % 4)
     return FG_ERR_ARG;
-  attn_tile_kernel<<<dim3(n_items, n_kv), 256, 0, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
-      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window);
+#define LAUNCH(PERM)                                                                                        \
+  attn_tile_kernel<PERM><<<dim3(n_items, n_kv), 256, 0, stream>>>(                                          \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
+      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
+  if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
+#undef LAUNCH
   return fg_launch_status();
 }
 

@@ -18,25 +18,30 @@
 #pragma once
 
 struct KvLayout {
-  int page_size, hd, kb, db, permuted;
+  int page_size, hd, kb_shift, db_shift, permuted;  // KB = 1 << kb_shift, DB = 1 << db_shift
   __host__ __device__ KvLayout(int P, int head_dim)
-      : page_size(P), hd(head_dim), kb(P % 16 == 0 ? 16 : 8), db(head_dim % 16 == 0 ? 16 : 8),
+      : page_size(P), hd(head_dim), kb_shift(P % 16 == 0 ? 4 : 3), db_shift(head_dim % 16 == 0 ? 4 : 3),
         permuted(P % 32 == 0) {}
   // element offset of (key kappa in page, head dim d) in the page's K part of one kv head
   __host__ __device__ size_t k_off(int kappa, int d) const {
-    return ((size_t)((kappa / kb) * (hd / 8) + d / 8) * kb + kappa % kb) * 8 + d % 8;
+    const int kb = 1 << kb_shift;
+    return ((size_t)(((kappa >> kb_shift) * (hd >> 3) + (d >> 3)) << kb_shift) + (kappa & (kb - 1))) * 8 + (d & 7);
   }
   __host__ __device__ int v_slot(int kappa) const {
     if (!permuted) return kappa;
-    const int k = kappa % 32;
-    return kappa - k + 8 * ((k % 16) / 4) + 4 * (k / 16) + k % 4;
+    const int k = kappa & 31;
+    return kappa - k + 8 * ((k & 15) >> 2) + 4 * (k >> 4) + (k & 3);
   }
   __host__ __device__ size_t v_off(int kappa, int d) const {
     const int s = v_slot(kappa);
-    return ((size_t)((d / db) * (page_size / 8) + s / 8) * db + d % db) * 8 + s % 8;
+    return v_chunk_off(s >> 3, d) + (s & 7);
   }
   // first element of the chunk (dim d, key chunk kc)
   __host__ __device__ size_t v_chunk_off(int kc, int d) const {
-    return ((size_t)((d / db) * (page_size / 8) + kc) * db + d % db) * 8;
+    const int db = 1 << db_shift;
+    return ((size_t)(((d >> db_shift) * (page_size >> 3) + kc) << db_shift) + (d & (db - 1))) * 8;
   }
+  // elements between the same chunk of consecutive 32-dim steps of K / consecutive dim blocks of V
+  __host__ __device__ size_t k_step32() const { return (size_t)32 << kb_shift; }
+  __host__ __device__ size_t v_step_block() const { return (size_t)(page_size >> 3) << (db_shift + 3); }
 };
