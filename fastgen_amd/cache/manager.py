@@ -158,6 +158,17 @@ class CacheManager:
     def n_table_entries(self, rid: Hashable, group: int = 0) -> int:
         return len(self._live[rid].pages[group])
 
+    def pages_of(self, rid: Hashable, group: int = 0) -> List[int]:
+        """The request's own page list (not a copy; do not change it)."""
+        return self._live[rid].pages[group]
+
+    def write_slot(self, rid: Hashable, group: int, pos: int) -> int:
+        """:meth:`write_slots` for one position."""
+        page = self._live[rid].pages[group][pos // self.page_size]
+        if page < 0:
+            raise RuntimeError(f"request {rid!r}: position in a released page of group {group}")
+        return page * self.page_size + pos % self.page_size
+
     def write_slots(self, rid: Hashable, group: int, start: int, n: int) -> np.ndarray:
         """Flat token slots ``page*page_size + offset`` of positions
         ``start .. start+n-1`` (which must be reserved)."""

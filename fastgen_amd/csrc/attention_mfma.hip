@@ -96,31 +96,39 @@ struct ItemRows {
 //   load_k(kb, ks) -> bf16x8 : K[16*kb + lane%16][32*ks + 8*(lane/16) ..+7]
 //   load_v(db, ks) -> bf16x8 : V^T[16*db + lane%16][the 8 keys 32*ks + 4g + i, 32*ks + 16 + 4g + i]
 //                              with g = lane/16, i = 0..3: the keys of pop[ks]
-template <class LK, class LV>
+// PREFETCH: operands come from memory; all of K and half of V are requested
+// before anything is computed (more registers).  Otherwise (operands in LDS)
+// each is read where it is used.
+template <bool PREFETCH, class LK, class LV>
 __device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf16x8 (&qop)[NKS], float scale,
                                             float& m, float& l, f32x4 (&o)[NDB], LK load_k, LV load_v) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
   // The order of the loads in the source is the order in which they are issued: all of K, then the
   // first half of V, are in flight before the first MFMA waits for anything; the second half of V is
   // issued when K's registers are free and flies during the softmax.
-  bf16x8 kop[4][NKS];
+  bf16x8 kop[PREFETCH ? 4 : 1][NKS];
+  bf16x8 vop0[PREFETCH ? NDB : 1], vop1[PREFETCH ? NDB : 1];
+  if (PREFETCH) {
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
+    for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) kop[kb][ks] = load_k(kb, ks);
-  bf16x8 vop0[NDB], vop1[NDB];
+      for (int ks = 0; ks < NKS; ++ks) kop[kb][ks] = load_k(kb, ks);
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) vop0[db] = load_v(db, 0);
+    for (int db = 0; db < NDB; ++db) vop0[db] = load_v(db, 0);
+  }
   f32x4 s[4];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
     s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
-      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[kb][ks], qop[ks], s[kb], 0, 0, 0);
+      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? kop[kb][ks] : load_k(kb, ks), qop[ks], s[kb], 0,
+                                                      0, 0);
   }
+  if (PREFETCH) {
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) vop1[db] = load_v(db, 1);
+    for (int db = 0; db < NDB; ++db) vop1[db] = load_v(db, 1);
+  }
   float mx = -INFINITY;
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb)
@@ -151,11 +159,11 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf
 #pragma unroll
   for (int db = 0; db < NDB; ++db) {
     o[db] *= alpha;
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop0[db], pop[0], o[db], 0, 0, 0);
+    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? vop0[db] : load_v(db, 0), pop[0], o[db], 0, 0, 0);
   }
 #pragma unroll
   for (int db = 0; db < NDB; ++db)
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop1[db], pop[1], o[db], 0, 0, 0);
+    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? vop1[db] : load_v(db, 1), pop[1], o[db], 0, 0, 0);
 }
 
 // qrow is always a readable row; `valid` says whether it is this lane's
@@ -265,7 +273,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
       }
       return and_mask(v, vmask[ks]);
     };
-    attend_tile(k0, me, qop, scale, m, l, o, load_k, load_v);
+    attend_tile<true>(k0, me, qop, scale, m, l, o, load_k, load_v);
   }
   l += __shfl_xor(l, 16, FG_WAVE);
   l += __shfl_xor(l, 32, FG_WAVE);
@@ -424,22 +432,29 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   for (int db = 0; db < NDB; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const size_t head_elems = (size_t)page_size * HD;
-  constexpr int KCH = HD / 8;  // 16-byte chunks in a key
-  for (int k0 = (first_min / TILE) * TILE; k0 <= pos_last; k0 += TILE) {
-    __syncthreads();  // the previous tile is no longer read
-    // (loads are never conditional: addresses are clamped into the item's key range, what lies
-    // outside is masked; keys beyond the range give scores that the select discards)
+  constexpr int KCH = HD / 8;                  // 16-byte chunks in a key
+  constexpr int KTOT = TILE * KCH, VTOT = NDB * 8 * 16;  // chunks of a K tile, of a V tile
+  constexpr int KN = (KTOT + 255) / 256;       // K chunks a thread copies per tile
+  constexpr int VN = (VTOT + 255) / 256;       // V chunks a thread copies per tile
+  bf16x8 kreg[KN], vreg[VN];
+  // The next tile's chunks are fetched into registers while the current tile is computed from
+  // LDS.  Loads are never conditional: addresses are clamped into the item's key range, value
+  // slots outside it are masked, keys outside it give scores that the select discards.
+  auto fetch = [&](int k0) {
     // K: chunk (block kb, dims 8c.., key r) -> k_s[((kb*KCH + c)*16 + r)*8]; r fastest over threads
-    for (int w = threadIdx.x; w < TILE * KCH; w += 256) {
+#pragma unroll
+    for (int j = 0; j < KN; ++j) {
+      const int w = min(threadIdx.x + 256 * j, KTOT - 1);  // beyond the tile: a copy that is not stored
       const int r = w & 15, c = (w >> 4) % KCH, kb = (w >> 4) / KCH;
       const int key = min(max(k0 + 16 * kb + r, first_min), pos_last);
-      *(bf16x8*)(k_s + (size_t)w * 8) =
-          *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
-                           lay.k_off(pager.in_page(key), 8 * c));
+      kreg[j] = *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                                 lay.k_off(pager.in_page(key), 8 * c));
     }
     // V: chunk (dim block db, key chunk kc = 4*ks + gg, dim r) -> v_s[((db*8 + kc)*16 + r)*8];
     // its slots are keys 32*ks + 4*gg + (0..3) and 16 more on
-    for (int w = threadIdx.x; w < NDB * 8 * 16; w += 256) {
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const int w = min(threadIdx.x + 256 * j, VTOT - 1);
       const int r = w & 15, kc = (w >> 4) & 7, db = w >> 7;
       const int ka = k0 + 32 * (kc >> 2) + 4 * (kc & 3), kb2 = ka + 16;
       const bool in_a = ka + 3 >= first_min && ka <= pos_last;
@@ -463,10 +478,21 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
           v[4 + e] = hi[e];
         }
       }
-      v = and_mask(v, slot_mask(ka, first_min, pos_last));
-      *(bf16x8*)(v_s + (size_t)w * 8) = v;
+      vreg[j] = and_mask(v, slot_mask(ka, first_min, pos_last));
     }
+  };
+  const int k_first = (first_min / TILE) * TILE;
+  fetch(k_first);
+  for (int k0 = k_first; k0 <= pos_last; k0 += TILE) {
+    __syncthreads();  // the previous tile is no longer read
+#pragma unroll
+    for (int j = 0; j < KN; ++j)
+      if (threadIdx.x + 256 * j < KTOT) *(bf16x8*)(k_s + (size_t)(threadIdx.x + 256 * j) * 8) = kreg[j];
+#pragma unroll
+    for (int j = 0; j < VN; ++j)
+      if (threadIdx.x + 256 * j < VTOT) *(bf16x8*)(v_s + (size_t)(threadIdx.x + 256 * j) * 8) = vreg[j];
     __syncthreads();
+    if (k0 + TILE <= pos_last) fetch(k0 + TILE);  // flies during this tile's MFMAs
     if (k0 > w_hi || k0 + TILE <= w_lo) continue;  // nothing in this tile for this wave's rows
     auto load_k = [&](int kb, int ks) -> bf16x8 {
       const int c = 4 * ks + g;
@@ -475,7 +501,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
     auto load_v = [&](int db, int ks) -> bf16x8 {
       return *(const bf16x8*)(v_s + ((db * 8 + 4 * ks + g) * 16 + r16) * 8);
     };
-    attend_tile(k0, me, qop, scale, m, l, o, load_k, load_v);
+    attend_tile<false>(k0, me, qop, scale, m, l, o, load_k, load_v);
   }
   l += __shfl_xor(l, 16, FG_WAVE);
   l += __shfl_xor(l, 32, FG_WAVE);

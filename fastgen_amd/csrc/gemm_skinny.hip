@@ -1,0 +1,226 @@
+// y = x W^T for few rows of x (decode: M <= 64), bf16 operands, fp32
+// accumulation on the matrix cores.  The work is streaming W once from HBM,
+// so the kernel is built around keeping many 16-byte loads of W in flight:
+//
+//  * a workgroup owns 16 rows of W (16 output columns); its waves split K,
+//    each wave walks its K range with v_mfma_f32_16x16x32_bf16 taking W as
+//    the A operand (16 rows x 32 k) and x^T as B (32 k x 16 rows of x), eight
+//    k steps unrolled so that 8 loads of W per lane are in flight; x (a few
+//    KB per k range) comes from the caches;
+//  * the waves' partial 16x16 tiles are added in LDS in wave order, so a
+//    result does not depend on timing;
+//  * the epilogue stores bf16 or fp32, or, for a gate/up matrix whose rows are
+//    interleaved in groups of 8 (8 gate rows, then their 8 up rows), stores
+//    silu(gate) * up directly: the gate/up activations never reach memory.
+//
+// Replaces the library product of fastgen/forward.py:433-513 where M is small.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define EPI_STORE 0
+#define EPI_SILU_MUL 1
+
+__device__ __forceinline__ bf16x8 gs_zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+template <int MB, int WAVES, int EPI, class TY>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
+    int ldy, int M, int N, int K) {
+  constexpr int U = MB <= 2 ? 8 : 4;  // k steps in flight
+  __shared__ float red[WAVES][MB * 256];
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  // rows are clamped, not skipped: what they give is not stored
+  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const bf16_t* xrow[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) xrow[mb] = x + (size_t)min(16 * mb + r16, M - 1) * ldx;
+
+  const int kw = ((K + WAVES * 32 - 1) / (WAVES * 32)) * 32;  // k per wave
+  const int k_begin = min(K, wave * kw), k_end = min(K, k_begin + kw);
+  f32x4 acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kk = k_begin; kk < k_end; kk += 32 * U) {
+    bf16x8 a[U], b[U][MB];
+    // all loads first, unconditional (addresses clamped), so that they are issued together
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = kk + 32 * u + 8 * g;
+      const bool in = k < k_end;  // K % 8 == 0: a chunk is inside or outside as a whole
+      const int kc = in ? k : k_begin;
+      const bf16x8 av = *(const bf16x8*)(wrow + kc);
+      a[u] = in ? av : gs_zero8();
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) b[u][mb] = *(const bf16x8*)(xrow[mb] + kc);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mb], acc[mb], 0, 0, 0);
+  }
+  // acc[mb][i] = C[n = 4g + i][m = 16 mb + r16]
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) *(f32x4*)(&red[wave][(mb * 16 + r16) * 16 + 4 * g]) = acc[mb];
+  __syncthreads();
+  if (EPI == EPI_STORE) {
+    for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
+      float s = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) s += red[wv][e];
+      const int m = e >> 4, n = n0 + (e & 15);
+      if (m < M && n < N) y[(size_t)m * ldy + n] = from_f<TY>(s);
+    }
+  } else {
+    // rows n0 .. n0+7 are gate rows j0 .. j0+7, rows n0+8 .. n0+15 their up rows; j0 = n0 / 2
+    for (int e = threadIdx.x; e < MB * 128; e += WAVES * 64) {
+      const int m = e >> 3, j = e & 7;
+      float gate = 0.f, up = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        gate += red[wv][m * 16 + j];
+        up += red[wv][m * 16 + 8 + j];
+      }
+      const int col = n0 / 2 + j;
+      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + col] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+    }
+  }
+}
+
+// The same for at most 16 rows of x with x going through LDS: a lane of an
+// MFMA operand row group reads 16 different rows of x, which from memory is 16
+// cache lines for 256 bytes; instead the wave copies its 16 x 256 slice of x
+// for the next 8 k steps with whole-row loads into LDS, chunk-major, and reads
+// the operands from there (the 16 lanes then read 256 contiguous bytes).
+template <int WAVES, int EPI, class TY>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
+    const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
+    int ldy, int M, int N, int K) {
+  constexpr int U = 8;
+  __shared__ float red[WAVES][256];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[WAVES][4 * U * 16 * 8];  // [k chunk][row][8]
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const int kw = ((K + WAVES * 32 - 1) / (WAVES * 32)) * 32;
+  const int k_begin = min(K, wave * kw), k_end = min(K, k_begin + kw);
+  // copying x: a row's 256 k of one iteration are 32 chunks = 32 lanes; a load covers 2 rows
+  const int c_row = lane >> 5, c_chunk = lane & 31;
+  const int x_loads = (M + 1) / 2;
+  bf16_t* my_xs = xs[wave];
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kk = k_begin; kk < k_end; kk += 32 * U) {
+    bf16x8 a[U], xv[8];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = kk + 32 * u + 8 * g;
+      const bool in = k < k_end;
+      const bf16x8 av = *(const bf16x8*)(wrow + (in ? k : k_begin));
+      a[u] = in ? av : gs_zero8();
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (j < x_loads) {  // uniform
+        const int row = min(2 * j + c_row, M - 1), k = kk + 8 * c_chunk;
+        xv[j] = *(const bf16x8*)(x + (size_t)row * ldx + (k < k_end ? k : k_begin));
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // the reads of the previous iteration are done (same wave, in order)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < x_loads) *(bf16x8*)(my_xs + (c_chunk * 16 + 2 * j + c_row) * 8) = xv[j];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bf16x8 b = *(const bf16x8*)(my_xs + ((4 * u + g) * 16 + r16) * 8);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc, 0, 0, 0);
+    }
+  }
+  *(f32x4*)(&red[wave][r16 * 16 + 4 * g]) = acc;
+  __syncthreads();
+  if (EPI == EPI_STORE) {
+    for (int e = threadIdx.x; e < 256; e += WAVES * 64) {
+      float s = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) s += red[wv][e];
+      const int m = e >> 4, n = n0 + (e & 15);
+      if (m < M && n < N) y[(size_t)m * ldy + n] = from_f<TY>(s);
+    }
+  } else {
+    for (int e = threadIdx.x; e < 128; e += WAVES * 64) {
+      const int m = e >> 3, j = e & 7;
+      float gate = 0.f, up = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        gate += red[wv][m * 16 + j];
+        up += red[wv][m * 16 + 8 + j];
+      }
+      if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + n0 / 2 + j] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+    }
+  }
+}
+
+template <int MB, int EPI, class TY>
+static void launch_skinny(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
+                          int K, hipStream_t stream) {
+  const int blocks = (N + 15) / 16;
+  if (MB == 1 && M > 1) {  // one row of x is a broadcast already
+    if (blocks >= 1024)
+      gemm_skinny16_kernel<4, EPI, TY><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
+                                                                   (TY*)y, ldy, M, N, K);
+    else
+      gemm_skinny16_kernel<8, EPI, TY><<<blocks, 512, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
+                                                                   (TY*)y, ldy, M, N, K);
+    return;
+  }
+  // few blocks: more waves a block, so that enough loads are in flight on every CU
+  if (blocks >= 1024)
+    gemm_skinny_kernel<MB, 4, EPI, TY><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
+                                                                   (TY*)y, ldy, M, N, K);
+  else
+    gemm_skinny_kernel<MB, 8, EPI, TY><<<blocks, 512, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
+                                                                   (TY*)y, ldy, M, N, K);
+}
+
+// x [M, K] bf16 (M <= 64), w [N, K] bf16, K % 8 == 0, rows 16-byte aligned.
+// epilogue 0: y [M, N] of out_dtype; epilogue 1: w's rows interleaved gate/up in
+// groups of 8 (N % 16 == 0), y [M, N/2] = silu(gate) * up of out_dtype.
+extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
+                              int K, int out_dtype, int epilogue, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return FG_OK;
+  if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return FG_ERR_ARG;
+  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2)) return FG_ERR_ARG;
+  if (epilogue == EPI_STORE && ldy < N) return FG_ERR_ARG;
+  if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
+  const int mb = (M + 15) / 16;
+#define GO(MB)                                                                                        \
+  do {                                                                                                \
+    if (epilogue == EPI_STORE && out_dtype == FG_BF16)                                                \
+      launch_skinny<MB, EPI_STORE, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, stream);                  \
+    else if (epilogue == EPI_STORE && out_dtype == FG_F32)                                            \
+      launch_skinny<MB, EPI_STORE, float>(x, ldx, w, ldw, y, ldy, M, N, K, stream);                   \
+    else if (epilogue == EPI_SILU_MUL && out_dtype == FG_BF16)                                        \
+      launch_skinny<MB, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, stream);               \
+    else                                                                                              \
+      return FG_ERR_ARG;                                                                              \
+  } while (0)
+  if (mb == 1) GO(1);
+  else if (mb == 2) GO(2);
+  else if (mb == 3) GO(3);
+  else GO(4);
+#undef GO
+  return fg_launch_status();
+}

@@ -17,10 +17,33 @@
 
 #define ROPE_THREADS 256
 
+// cos and sin of float(pos) * freqs[i] for every token of the step, computed
+// once and shared by all layers: table[(t * n_freqs + i) * 2 + {0, 1}].
+__global__ __launch_bounds__(ROPE_THREADS) void rope_table_kernel(
+    const int* __restrict__ positions, const float* __restrict__ freqs, float* __restrict__ table,
+    int n_tokens, int n_freqs) {
+  const int e = blockIdx.x * ROPE_THREADS + threadIdx.x;
+  if (e >= n_tokens * n_freqs) return;
+  const float ang = (float)positions[e / n_freqs] * freqs[e % n_freqs];
+  table[2 * e] = cosf(ang);
+  table[2 * e + 1] = sinf(ang);
+}
+
+extern "C" int fg_rope_table(const int* positions, const float* freqs, float* table, int n_tokens,
+                             int n_freqs, hipStream_t stream) {
+  if (n_tokens <= 0 || n_freqs <= 0) return FG_OK;
+  const long long n = (long long)n_tokens * n_freqs;
+  if (n > 2147483647LL) return FG_ERR_ARG;
+  rope_table_kernel<<<(unsigned)((n + ROPE_THREADS - 1) / ROPE_THREADS), ROPE_THREADS, 0, stream>>>(
+      positions, freqs, table, n_tokens, n_freqs);
+  return fg_launch_status();
+}
+
 template <class T>
 __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
     T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
-    const float* __restrict__ freqs, const int* __restrict__ slots, T* __restrict__ k_pages,
+    const float* __restrict__ freqs, const float* __restrict__ table, const int* __restrict__ slots,
+    T* __restrict__ k_pages,
     T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
     int write_kv) {
   const int t = blockIdx.x;
@@ -41,8 +64,15 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
     T* x = row + (size_t)head * hd + 2 * i;
     float a = to_f<T>(x[0]), b = to_f<T>(x[1]);
     if (2 * i < rotary_dim) {
-      const float ang = pos * freqs[i];
-      const float s = sinf(ang), c = cosf(ang);
+      float s, c;
+      if (table) {
+        c = table[((size_t)t * (rotary_dim / 2) + i) * 2];
+        s = table[((size_t)t * (rotary_dim / 2) + i) * 2 + 1];
+      } else {
+        const float ang = pos * freqs[i];
+        s = sinf(ang);
+        c = cosf(ang);
+      }
       const float ra = a * c - b * s;
       const float rb = b * c + a * s;
       a = ra;
@@ -72,7 +102,8 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_kernel(
 template <class T>
 __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
     T* __restrict__ qkv, int row_stride, const int* __restrict__ positions,
-    const float* __restrict__ freqs, const int* __restrict__ slots, T* __restrict__ k_pages,
+    const float* __restrict__ freqs, const float* __restrict__ table, const int* __restrict__ slots,
+    T* __restrict__ k_pages,
     T* __restrict__ v_pages, int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
     int write_kv) {
   const int t = blockIdx.x;
@@ -94,10 +125,20 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
       float v[8];
       load8<T>(x, v);
       if (8 * c < rotary_dim) {
+        float cs4[8];  // cos, sin of the chunk's four pairs
+        if (table) {
+          load8<float>(table + ((size_t)t * (rotary_dim / 2) + 4 * c) * 2, cs4);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float ang = pos * freqs[4 * c + j];
+            cs4[2 * j] = cosf(ang);
+            cs4[2 * j + 1] = sinf(ang);
+          }
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float ang = pos * freqs[4 * c + j];
-          const float sn = sinf(ang), cs = cosf(ang);
+          const float cs = cs4[2 * j], sn = cs4[2 * j + 1];
           const float a = v[2 * j], b = v[2 * j + 1];
           v[2 * j] = a * cs - b * sn;
           v[2 * j + 1] = b * cs + a * sn;
@@ -120,8 +161,10 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
 // qkv: [n_tokens, row_stride] with q heads, then k heads, then v heads in a
 // row.  With write_kv == 0 only q is rotated (a mixer that reads another
 // layer's cache).
+// `table` (from fg_rope_table, for the same positions) replaces the sin/cos
+// of `freqs` when given.
 extern "C" int fg_rope_kv_write(void* qkv, int row_stride, const int* positions,
-                                const float* freqs, const int* slots, void* k_pages,
+                                const float* freqs, const float* table, const int* slots, void* k_pages,
                                 void* v_pages, int n_tokens, int n_heads, int n_kv, int hd,
                                 int rotary_dim, int page_size, int write_kv, int dtype,
                                 hipStream_t stream) {
@@ -133,9 +176,9 @@ extern "C" int fg_rope_kv_write(void* qkv, int row_stride, const int* positions,
   if (row_stride < (n_heads + (write_kv ? 2 * n_kv : 0)) * hd) return FG_ERR_ARG;
   const bool vec = hd % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0;
 #define LAUNCH(T, KERNEL)                                                                         \
-  KERNEL<T><<<n_tokens, ROPE_THREADS, 0, stream>>>((T*)qkv, row_stride, positions, freqs, slots, \
-                                                   (T*)k_pages, (T*)v_pages, n_heads, n_kv, hd,  \
-                                                   rotary_dim, page_size, write_kv)
+  KERNEL<T><<<n_tokens, ROPE_THREADS, 0, stream>>>((T*)qkv, row_stride, positions, freqs, table,  \
+                                                   slots, (T*)k_pages, (T*)v_pages, n_heads, n_kv, \
+                                                   hd, rotary_dim, page_size, write_kv)
   if (dtype == FG_F32) {
     if (vec) LAUNCH(float, rope_kv_write_vec_kernel); else LAUNCH(float, rope_kv_write_kernel);
   } else if (dtype == FG_BF16) {

@@ -194,17 +194,20 @@ extern "C" int fg_rmsnorm(const void* x, const void* w, void* out, int n_rows, i
 }
 
 // ------------------------------------------------------------- SiLU(g) * u
-// gu is [n_rows, 2*hidden]: the gate columns first, then the up columns.
+// gu is [n_rows, 2*hidden] with gate and up columns interleaved in groups of
+// 8: columns 16k .. 16k+7 are gate 8k .. 8k+7, columns 16k+8 .. 16k+15 their up
+// values (the row order in which the gate/up matrix is kept, so that one tile
+// of a matrix product holds both).  hidden % 8 == 0.
 template <class TA>
 __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_kernel(
     const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
-  const TA* g = gu + (size_t)blockIdx.y * 2 * hidden;
-  const TA* u = g + hidden;
+  const TA* row = gu + (size_t)blockIdx.y * 2 * hidden;
   TA* o = out + (size_t)blockIdx.y * hidden;
   const int i = blockIdx.x * ROWS_THREADS + threadIdx.x;
   if (i < hidden) {
-    const float gv = to_f<TA>(g[i]);
-    const float uv = to_f<TA>(u[i]);
+    const int col = 16 * (i / 8) + i % 8;
+    const float gv = to_f<TA>(row[col]);
+    const float uv = to_f<TA>(row[col + 8]);
     o[i] = from_f<TA>(gv / (1.f + expf(-gv)) * uv);
   }
 }
@@ -213,14 +216,13 @@ __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_kernel(
 template <class TA>
 __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_vec_kernel(
     const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
-  const TA* g = gu + (size_t)blockIdx.y * 2 * hidden;
-  const TA* u = g + hidden;
+  const TA* row = gu + (size_t)blockIdx.y * 2 * hidden;
   TA* o = out + (size_t)blockIdx.y * hidden;
   const int e = (blockIdx.x * ROWS_THREADS + threadIdx.x) * 8;
   if (e < hidden) {
     float gv[8], uv[8], r[8];
-    load8<TA>(g + e, gv);
-    load8<TA>(u + e, uv);
+    load8<TA>(row + 2 * e, gv);
+    load8<TA>(row + 2 * e + 8, uv);
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = gv[i] / (1.f + expf(-gv[i])) * uv[i];
     store8<TA>(o + e, r);
@@ -230,11 +232,11 @@ __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_vec_kernel(
 extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, int act_dtype,
                            hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
-  if (hidden <= 0 || n_rows > 65535 * 32) return FG_ERR_ARG;
+  if (hidden <= 0 || hidden % 8 || n_rows > 65535 * 32) return FG_ERR_ARG;
   // blockIdx.y is limited to 65535: rows beyond that go to further launches
   for (int r0 = 0; r0 < n_rows; r0 += 65535) {
     const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
-    const bool vec = hidden % 8 == 0;
+    const bool vec = true;  // hidden % 8 == 0 is required by the interleaved layout
     const int per_block = vec ? ROWS_THREADS * 8 : ROWS_THREADS;
     dim3 grid((hidden + per_block - 1) / per_block, nr);
     if (act_dtype == FG_F32) {

@@ -105,7 +105,7 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
               (n_cached + q_lens).astype(np.int32), slot_ids, np.asarray(out_rows, dtype=np.int32)]
     table_shapes = []
     for g in range(cache.n_groups):
-        width = max(cache.n_table_entries(e.rid, g) for e in entries)
+        width = max(len(cache.pages_of(e.rid, g)) for e in entries)
         if table_width is not None:
             if width > table_width:
                 raise ValueError(f"a request holds {width} pages, the fixed table width is {table_width}")
@@ -113,9 +113,12 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
         tbl = np.zeros((B, max(1, width)), dtype=np.int32)
         slots = np.empty(T, dtype=np.int32)
         for b, e in enumerate(entries):
-            row = cache.block_table(e.rid, g)
+            row = cache.pages_of(e.rid, g)
             tbl[b, : len(row)] = row
-            slots[q_start[b] : q_start[b + 1]] = cache.write_slots(e.rid, g, int(n_cached[b]), int(q_lens[b]))
+            if q_lens[b] == 1:
+                slots[q_start[b]] = cache.write_slot(e.rid, g, int(n_cached[b]))
+            else:
+                slots[q_start[b] : q_start[b + 1]] = cache.write_slots(e.rid, g, int(n_cached[b]), int(q_lens[b]))
         table_shapes.append(tbl.shape)
         pieces += [tbl.reshape(-1), slots]
     offs = np.cumsum([0] + [p.size for p in pieces])

@@ -76,7 +76,7 @@ class Engine:
         if plan:
             entries, rows = [], []
             for e in plan:
-                toks = e.request.all_tokens()[e.start : e.start + e.n]
+                toks = e.request.tokens_from(e.start, e.n)
                 entries.append(StepEntry(e.request.rid, toks, [e.n - 1] if e.wants_logits else []))
                 if e.wants_logits:
                     rows.append(e.request)

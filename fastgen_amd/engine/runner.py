@@ -50,6 +50,9 @@ class _DecodeGraph:
             model.forward(self.ctx, runner.stores)
         torch.cuda.current_stream(model.device).wait_stream(side)
         torch.cuda.synchronize(model.device)
+        # what the warm-up derived from this step's values (tables of sines, ...) is derived again
+        # inside the capture, so that a replay derives it from its own values
+        self.ctx.scratch.clear()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, pool=runner.graph_pool):
             self.logits = model.forward(self.ctx, runner.stores)

@@ -30,7 +30,7 @@ from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
 from ..cache.manager import CacheManager
 
 
-@dataclass
+@dataclass(eq=False)  # requests are compared by identity: two with equal fields are still two
 class Request:
     rid: Hashable
     prompt: List[int]
@@ -49,6 +49,15 @@ class Request:
     def all_tokens(self) -> List[int]:
         return self.prompt + self.generated
 
+    def tokens_from(self, start: int, n: int) -> List[int]:
+        """``all_tokens()[start:start+n]`` without building the whole list."""
+        np_ = len(self.prompt)
+        if start >= np_:
+            return self.generated[start - np_ : start - np_ + n]
+        if start + n <= np_:
+            return self.prompt[start : start + n]
+        return self.prompt[start:] + self.generated[: start + n - np_]
+
     def n_known(self) -> int:
         return len(self.prompt) + len(self.generated)
 
@@ -58,7 +67,7 @@ class Request:
         return self.n_known() - self.n_fed
 
 
-@dataclass
+@dataclass(eq=False)
 class PlannedEntry:
     request: Request
     start: int  # index into all_tokens()
@@ -128,35 +137,39 @@ class Scheduler:
     def plan(self) -> List[PlannedEntry]:
         entries: List[PlannedEntry] = []
         budget = self.max_step_tokens
+        gone = set()  # ids of requests preempted or ended while planning
         # A. one token for every decoding request, oldest first; make room by
         #    preempting the youngest
         for req in list(self.running):
             if budget == 0:
                 break
-            if req not in self.running or req.remaining() != 1:
+            if id(req) in gone or req.remaining() != 1:
                 continue
             while not self.cache.can_reserve(req.rid, 1):
                 victim = self.running[-1]
                 if victim is req and len(self.running) == 1:
                     self._finish(req, "cache_full")
+                    gone.add(id(req))
                     break
                 # an entry already planned for the victim is withdrawn
                 entries = [e for e in entries if e.request is not victim]
                 self._preempt(victim)
+                gone.add(id(victim))
                 if victim is req:
                     break
-            if req not in self.running:
+            if id(req) in gone:
                 continue
             self.cache.reserve(req.rid, 1)
             entries.append(PlannedEntry(req, req.n_fed, 1, True))
             budget -= 1
         budget = self.max_step_tokens - sum(e.n for e in entries)
+        planned = {id(e.request) for e in entries}
         # B. portions of prompts already admitted, oldest first
         for req in self.running:
             if budget == 0:
                 break
             rem = req.remaining()
-            if rem < 1 or any(e.request is req for e in entries):
+            if rem < 1 or id(req) in planned:
                 continue
             n = self._fits(req, min(rem, budget))
             if n < 1:

@@ -41,6 +41,7 @@ LIBRARIES: Dict[str, str] = {
     "rope_kv": "rope_kv.hip",
     "attention": "attention.hip",
     "gemm": "gemm.hip",
+    "gemm_skinny": "gemm_skinny.hip",
     "sampling": "sampling.hip",
 }
 

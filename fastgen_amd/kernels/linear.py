@@ -1,9 +1,10 @@
 """``y = x W^T`` for the two precisions of the engine.
 
 float32: the engine's own fused-multiply-add kernel (``gemm.hip``), a true
-32-bit product whose rows do not depend on one another.  bfloat16: the
-vendor library's matrix product through ``torch`` (the reference uses cuBLAS
-through ``F.linear`` for the same products, ``fastgen/forward.py:433-513``),
+32-bit product whose rows do not depend on one another.  bfloat16: up to 64
+rows (decode) the engine's weight-streaming MFMA kernel (``gemm_skinny.hip``);
+more rows the vendor library's matrix product through ``torch`` (the reference
+uses cuBLAS through ``F.linear`` for all of them, ``fastgen/forward.py:433-513``),
 with fp32 accumulation; logits are asked for in fp32 directly.
 """
 
@@ -34,6 +35,13 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
         raise
 
 
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Few rows (decode): the engine's own weight-streaming kernel takes the product."""
+    return (x.dtype == torch.bfloat16 and x.shape[0] <= ops.SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+            and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     if not x.is_cuda:
         raise ops.KernelArgumentError("fastgen_amd runs on the GPU only; got a tensor on " + str(x.device))
@@ -44,6 +52,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return ops.gemm_nt(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
+    if skinny_ok(x, w):
+        return ops.gemm_skinny(x, w, out_dtype)
     if out_dtype == torch.bfloat16:
         return torch.nn.functional.linear(x, w)
     y = _library_mm_f32_out(x, w)

@@ -122,11 +122,25 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
     return out
 
 
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Rows of a gate and an up matrix ``[hidden, dim]`` as one matrix
+    ``[2*hidden, dim]`` in groups of 8: rows ``16k..16k+7`` are gate rows
+    ``8k..8k+7``, rows ``16k+8..16k+15`` the up rows of the same channels.  One
+    16-row tile of a product with it holds both halves of 8 channels, so
+    ``silu(gate) * up`` can be applied where the tile is stored."""
+    hidden, dim = gate.shape
+    _need(up.shape == gate.shape and hidden % 8 == 0,
+          f"gate and up must have the same shape and a row count that is a multiple of 8 (got {hidden})")
+    return torch.stack([gate.reshape(hidden // 8, 8, dim), up.reshape(hidden // 8, 8, dim)], dim=1).reshape(
+        2 * hidden, dim)
+
+
 def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(gate) * up`` of ``[T, 2*hidden]`` (gate columns first), fp32 inside."""
+    """``silu(gate) * up`` of ``[T, 2*hidden]`` whose columns are interleaved as
+    :func:`interleave_gate_up` orders the matrix rows; fp32 inside."""
     _gpu(gate_up, out)
-    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
-          "gate_up must be contiguous [T, 2*hidden]")
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 16 == 0,
+          "gate_up must be contiguous [T, 2*hidden] with hidden a multiple of 8")
     T, hidden = gate_up.shape[0], gate_up.shape[1] // 2
     out = torch.empty((T, hidden), dtype=gate_up.dtype, device=gate_up.device) if out is None else out
     _need(out.shape == (T, hidden) and out.dtype == gate_up.dtype and out.is_contiguous(), "out must be [T, hidden]")
@@ -136,10 +150,23 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
 
 
 # ------------------------------------------------------------ rope + kv write
+def rope_table(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """``[T, n_freqs, 2]`` fp32: cos and sin of ``float(pos) * freqs[i]``, for all
+    layers of a step that rotate with the same frequencies."""
+    _gpu(positions, freqs)
+    _i32(positions, "positions")
+    _need(freqs.dtype == torch.float32 and freqs.is_contiguous(), "freqs must be contiguous float32")
+    T, n = positions.numel(), freqs.numel()
+    table = torch.empty((T, n, 2), dtype=torch.float32, device=positions.device)
+    st = _lib.load("rope_kv").fg_rope_table(_ptr(positions), _ptr(freqs), _ptr(table), T, n, _stream(table))
+    _check(st, "rope_table")
+    return table
+
+
 def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[torch.Tensor],
                   slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
                   v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
-                  rotary_dim: int, write_kv: bool = True) -> None:
+                  rotary_dim: int, write_kv: bool = True, table: Optional[torch.Tensor] = None) -> None:
     """Rotate q and k of ``qkv [T, (H+2KV)*hd]`` in place and store k, v at
     ``slots`` of the paged cache (K pages ``[n_pages, KV, P, hd]``, V pages
     ``[n_pages, KV, hd, P]``).  ``kernels/rope.py:56-89``, ``forward.py:449-460``.
@@ -152,9 +179,12 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[to
     _i32(positions, "positions", T)
     _need(head_dim % 2 == 0 and 0 <= rotary_dim <= head_dim and rotary_dim % 2 == 0,
           "head_dim and rotary_dim must be even and rotary_dim <= head_dim")
-    if rotary_dim:
+    if rotary_dim and table is None:
         _need(freqs is not None and freqs.dtype == torch.float32 and freqs.is_contiguous()
               and freqs.numel() >= rotary_dim // 2, "freqs must be float32 [rotary_dim/2]")
+    if rotary_dim and table is not None:
+        _need(table.dtype == torch.float32 and table.is_contiguous() and table.shape == (T, rotary_dim // 2, 2),
+              "table must be float32 [T, rotary_dim/2, 2]")
     page_size = 1
     if write_kv:
         _need(slots is not None and k_pages is not None and v_pages is not None, "cache operands missing")
@@ -167,7 +197,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, freqs: Optional[to
               and v_pages.shape == (k_pages.shape[0], n_kv, head_dim, page_size),
               "v_pages must be contiguous [n_pages, KV, hd, P] of qkv's dtype")
     st = _lib.load("rope_kv").fg_rope_kv_write(
-        _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(freqs), _ptr(slots), _ptr(k_pages), _ptr(v_pages),
+        _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(freqs), _ptr(table if rotary_dim else None), _ptr(slots),
+        _ptr(k_pages), _ptr(v_pages),
         T, n_heads, n_kv, head_dim, rotary_dim, page_size, int(write_kv), _code(qkv), _stream(qkv))
     _check(st, "rope_kv_write")
 
@@ -342,6 +373,34 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
             _code(x), _code(out), _stream(out))
         _check(st, "gemm_nt")
     return out
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                silu_mul_epilogue: bool = False) -> torch.Tensor:
+    """``x @ w.T`` for at most 64 rows of bf16 ``x`` on the matrix cores, built to
+    stream ``w [N, K]`` once.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
+    ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
+    ``[M, N/2]``."""
+    _gpu(x, w)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16 operands")
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(0 < M <= SKINNY_MAX_ROWS, f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows, got {M}")
+    _need(K % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "K must be a multiple of 8, rows 16-byte aligned")
+    out_dtype = out_dtype or torch.bfloat16
+    if silu_mul_epilogue:
+        _need(N % 16 == 0 and out_dtype == torch.bfloat16, "the gate/up epilogue needs N % 16 == 0 and bf16 output")
+    y = torch.empty((M, N // 2 if silu_mul_epilogue else N), dtype=out_dtype, device=x.device)
+    st = _lib.load("gemm_skinny").fg_gemm_skinny(
+        _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, _code(y),
+        1 if silu_mul_epilogue else 0, _stream(x))
+    _check(st, "gemm_skinny")
+    return y
 
 
 # ------------------------------------------------------------------- sampling

@@ -49,8 +49,7 @@ class Attention(Mixer):
         wv = tensors[self._name("v_proj.weight")]
         self.wqkv = place(torch.cat([wq, wk, wv], dim=0), MATRIX, dtype, device)
         self.wo = place(tensors[self._name("o_proj.weight")], MATRIX, dtype, device)
-        f = self.position.frequencies()
-        self.freqs = None if f is None else f.to(device=device, dtype=torch.float32).contiguous()
+        self.freqs = self.position.frequencies_on(device)
 
     def paged_need(self) -> PagedNeed:
         return PagedNeed(self.n_kv_heads, self.head_dim, self.window)
@@ -61,9 +60,18 @@ class Attention(Mixer):
         # an entry that reads another entry's cache needs its queries only
         w = self.wqkv if store.owns else self.wqkv[:q_width]
         qkv = linear(x, w)
+        table = None
+        if self.freqs is not None:
+            # sin and cos of the step's positions: computed by the first layer, shared by all layers
+            # that rotate with the same frequencies
+            key = ("rope_table", self.freqs.data_ptr())
+            table = ctx.scratch.get(key)
+            if table is None:
+                table = ctx.scratch[key] = ops.rope_table(ctx.positions, self.freqs)
         ops.rope_kv_write(
             qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
             self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
+            table=table,
         )
         out = torch.empty((x.shape[0], q_width), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,

@@ -141,8 +141,22 @@ class PositionEncoding(Part):
     def frequencies(self) -> Optional[torch.Tensor]:
         return None
 
+    def frequencies_on(self, device: Any) -> Optional[torch.Tensor]:
+        """The frequency table on ``device``; parts with equal tables share one
+        tensor, so that what is derived from it per step is computed once."""
+        f = self.frequencies()
+        if f is None:
+            return None
+        key = (str(torch.device(device)), tuple(f.tolist()))
+        if key not in _FREQUENCY_TABLES:
+            _FREQUENCY_TABLES[key] = f.to(device=device, dtype=torch.float32).contiguous()
+        return _FREQUENCY_TABLES[key]
+
     def arrange_rows(self, w: torch.Tensor, n_heads: int) -> torch.Tensor:
         return w
+
+
+_FREQUENCY_TABLES: Dict[Tuple[str, Tuple[float, ...]], torch.Tensor] = {}
 
 
 # -------------------------------------------------------------- registries

@@ -1,6 +1,8 @@
 """Dense gated feed-forward (``fastgen/forward.py:483-499``):
-``down(silu(gate(x)) * up(x))``.  Gate and up are one matrix, so one product
-gives both."""
+``down(silu(gate(x)) * up(x))``.  Gate and up are one matrix with their rows
+interleaved in groups of 8, so one product gives both and a tile of it holds
+both halves of a channel: for few rows ``silu(gate) * up`` is applied where the
+product is stored."""
 
 from __future__ import annotations
 
@@ -9,7 +11,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear
+from ..kernels.linear import linear, skinny_ok
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
@@ -30,11 +32,17 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
         gate, up = tensors[self._name("gate_proj.weight")], tensors[self._name("up_proj.weight")]
-        self.w_gate_up = place(torch.cat([gate, up], dim=0), MATRIX, dtype, device)
+        if self.hidden_dim % 8:
+            raise ValueError(f"{self.prefix}: hidden_dim={self.hidden_dim} must be a multiple of 8")
+        self.w_gate_up = place(ops.interleave_gate_up(gate, up), MATRIX, dtype, device)
         self.w_down = place(tensors[self._name("down_proj.weight")], MATRIX, dtype, device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down)
+        if skinny_ok(x, self.w_gate_up):
+            act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True)
+        else:
+            act = ops.silu_mul(linear(x, self.w_gate_up))
+        return linear(act, self.w_down)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -83,21 +83,27 @@ def test_rmsnorm_per_head_rows(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,F", [(1, 14336), (9, 328), (70, 1000)])
+@pytest.mark.parametrize("T,F", [(1, 14336), (9, 328), (70, 1000), (3, 8)])
 def test_silu_mul(ops, dtype, T, F):
     torch.manual_seed(3)
-    gu = (torch.randn(T, 2 * F) * 4).to(dtype)
+    g, u = (torch.randn(T, F) * 4).to(dtype), (torch.randn(T, F) * 4).to(dtype)
+    # columns in groups of 8: 8 gate values, then the 8 up values of the same channels
+    gu = torch.stack([g.view(T, F // 8, 8), u.view(T, F // 8, 8)], dim=2).reshape(T, 2 * F).contiguous()
     got = ops.silu_mul(gu.to(DEV)).cpu()
-    g, u = gu[:, :F].float(), gu[:, F:].float()
-    want = (g * torch.sigmoid(g) * u).to(dtype)
+    want = (g.float() * torch.sigmoid(g.float()) * u.float()).to(dtype)
     assert torch.allclose(got.float(), want.float(), **tol(dtype))
+    # the same order for the rows of the weight matrix
+    wg, wu = torch.arange(F * 3.0).view(F, 3), -torch.arange(F * 3.0).view(F, 3)
+    w = ops.interleave_gate_up(wg, wu)
+    assert torch.equal(w[16:24], wg[8:16]) and torch.equal(w[24:32], wu[8:16])
 
 
 # ------------------------------------------------------------- rope + write
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,hd,rot,P", [(4, 2, 16, 16, 16), (5, 1, 48, 48, 32), (8, 8, 128, 128, 64),
                                            (6, 3, 64, 32, 8), (3, 3, 80, 0, 16)])
-def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P):
+@pytest.mark.parametrize("with_table", [False, True])
+def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P, with_table):
     torch.manual_seed(4)
     T, n_pages = 37, 9
     width = (H + 2 * KV) * hd
@@ -109,8 +115,13 @@ def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P):
     kp = torch.full((n_pages, KV, P, hd), 7.0, dtype=dtype)
     vp = torch.full((n_pages, KV, hd, P), 7.0, dtype=dtype)
     qkv_d, kp_d, vp_d = qkv.to(DEV), kp.to(DEV), vp.to(DEV)
+    table = None
+    if with_table and rot:  # sines and cosines computed once for the step, as the engine does
+        table = ops.rope_table(pos.to(DEV), freqs.to(DEV))
+        ang = pos.float()[:, None] * freqs[None, :]
+        assert torch.allclose(table.cpu(), torch.stack([torch.cos(ang), torch.sin(ang)], -1), atol=1e-6)
     ops.rope_kv_write(qkv_d, pos.to(DEV), None if freqs is None else freqs.to(DEV), slots.to(DEV), kp_d, vp_d,
-                      H, KV, hd, rot)
+                      H, KV, hd, rot, table=table)
     q = qkv[:, : H * hd].view(T, H, hd)
     k = qkv[:, H * hd : (H + KV) * hd].view(T, KV, hd)
     v = qkv[:, (H + KV) * hd :].view(T, KV, hd)
@@ -276,6 +287,49 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
     for rows in ([0], [69], list(range(3, 68))):
         part = ops.gemm_nt(x[rows].to(DEV), w.to(DEV)).cpu()
         assert torch.equal(part, full[rows])  # bit for bit
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(515, 240), (4096, 4096), (6144, 64), (48, 8), (1000, 14336), (16, 328)])
+@pytest.mark.parametrize("odtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny(ops, M, N, K, odtype):
+    torch.manual_seed(14)
+    x, w = torch.randn(M, K).bfloat16(), (torch.randn(N, K) * 0.1).bfloat16()
+    got = ops.gemm_skinny(x.to(DEV), w.to(DEV), out_dtype=odtype).cpu()
+    want = x.double() @ w.double().T
+    assert got.dtype == odtype and got.shape == (M, N)
+    err = (got.double() - want).abs().max() / want.abs().max()
+    assert err < (1e-5 if odtype == torch.float32 else 6e-3), float(err)
+
+
+def test_gemm_skinny_takes_views_and_refuses_the_rest(ops):
+    from fastgen_amd.kernels import KernelArgumentError
+
+    torch.manual_seed(15)
+    big = torch.randn(8, 3 * 256).bfloat16().to(DEV)
+    w = torch.randn(40, 256).bfloat16().to(DEV)
+    x = big[:, 256:512]  # a column slice: row stride 768
+    got = ops.gemm_skinny(x, w).cpu().float()
+    assert torch.allclose(got, x.cpu().float() @ w.cpu().float().T, atol=0.3, rtol=2e-2)
+    with pytest.raises(KernelArgumentError, match="rows"):
+        ops.gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    with pytest.raises(KernelArgumentError, match="multiple of 8"):
+        ops.gemm_skinny(torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV),
+                        torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("M", [1, 8, 40])
+@pytest.mark.parametrize("F,K", [(328, 240), (14336, 4096), (8, 64)])
+def test_gemm_skinny_gate_up_epilogue(ops, M, F, K):
+    torch.manual_seed(16)
+    x = torch.randn(M, K).bfloat16()
+    wg, wu = (torch.randn(F, K) * 0.05).bfloat16(), (torch.randn(F, K) * 0.05).bfloat16()
+    w = ops.interleave_gate_up(wg, wu).contiguous().to(DEV)
+    got = ops.gemm_skinny(x.to(DEV), w, silu_mul_epilogue=True).cpu().float()
+    g, u = x.float() @ wg.float().T, x.float() @ wu.float().T
+    want = g * torch.sigmoid(g) * u
+    assert got.shape == (M, F)
+    assert (got - want).abs().max() <= 1e-2 * want.abs().max() + 1e-3
 
 
 # ----------------------------------------------------------------- sampling
