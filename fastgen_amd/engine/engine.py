@@ -133,19 +133,28 @@ class Engine:
         """Seconds of exactly ``steps`` decode steps of the batch ``prompts``
         (greedy, no stop ids), after the prompts are in the cache and after
         ``warmup`` untimed decode steps."""
-        params = SamplingParams(temperature=0.0, max_new_tokens=warmup + steps + 1)
+        # the first requests decode while the later prompts are still being fed: none may end
+        # before the timed steps are over
+        n_prompt_tokens = sum(len(p) for p in prompts)
+        feed_steps = -(-n_prompt_tokens // max(1, self.scheduler.max_step_tokens - len(prompts))) + len(prompts)
+        params = SamplingParams(temperature=0.0, max_new_tokens=feed_steps + warmup + steps + 8)
         for p in prompts:
             self.add_request(p, params)
         while any(r.remaining() > 1 for r in self.scheduler.running) or self.scheduler.waiting:
             self.step()
         for _ in range(warmup):
             self.step()
+        if len(self.scheduler.running) != len(prompts) or self.scheduler.n_preemptions:
+            raise RuntimeError("time_decode: the batch did not stay whole; give the cache more pages")
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            self.step()
+            done = self.step()
+            if done:
+                raise RuntimeError("time_decode: a request ended inside the timed steps")
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        while self.has_work():
-            self.step()
+        for r in list(self.scheduler.running):  # the measurement is over: let go of the batch
+            self.scheduler._finish(r, "aborted")
+        self.scheduler.finished.clear()
         return dt

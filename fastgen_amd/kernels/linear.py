@@ -1,7 +1,7 @@
 """``y = x W^T`` for the two precisions of the engine.
 
 float32: the engine's own fused-multiply-add kernel (``gemm.hip``), a true
-32-bit product whose rows do not depend on one another.  bfloat16: up to 64
+32-bit product whose rows do not depend on one another.  bfloat16: up to 16
 rows (decode) the engine's weight-streaming MFMA kernel (``gemm_skinny.hip``);
 more rows the vendor library's matrix product through ``torch`` (the reference
 uses cuBLAS through ``F.linear`` for all of them, ``fastgen/forward.py:433-513``),
@@ -35,9 +35,13 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
         raise
 
 
+# up to this many rows the weight-streaming kernel is faster than the library's product
+SKINNY_ROWS = 16
+
+
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Few rows (decode): the engine's own weight-streaming kernel takes the product."""
-    return (x.dtype == torch.bfloat16 and x.shape[0] <= ops.SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
