@@ -98,10 +98,12 @@ struct ItemRows {
 //                              with g = lane/16, i = 0..3: the keys of pop[ks]
 // PREFETCH: operands come from memory; all of K and half of V are requested
 // before anything is computed (more registers).  Otherwise (operands in LDS)
-// each is read where it is used.
-template <bool PREFETCH, class LK, class LV>
-__device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf16x8 (&qop)[NKS], float scale,
-                                            float& m, float& l, f32x4 (&o)[NDB], LK load_k, LV load_v) {
+// each is read where it is used.  RB: blocks of 16 query rows a wave holds;
+// every K and V operand it reads serves all of them.
+template <bool PREFETCH, int RB, class LK, class LV>
+__device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], const bf16x8 (&qop)[RB][NKS],
+                                            float scale, float (&m)[RB], float (&l)[RB], f32x4 (&o)[RB][NDB],
+                                            LK load_k, LV load_v) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
   // The order of the loads in the source is the order in which they are issued: all of K, then the
   // first half of V, are in flight before the first MFMA waits for anything; the second half of V is
@@ -116,54 +118,64 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows& me, const bf
 #pragma unroll
     for (int db = 0; db < NDB; ++db) vop0[db] = load_v(db, 0);
   }
-  f32x4 s[4];
+  f32x4 s[RB][4];
 #pragma unroll
   for (int kb = 0; kb < 4; ++kb) {
-    s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks)
-      s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? kop[kb][ks] : load_k(kb, ks), qop[ks], s[kb], 0,
-                                                      0, 0);
+    for (int rb = 0; rb < RB; ++rb) s[rb][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const bf16x8 k = PREFETCH ? kop[kb][ks] : load_k(kb, ks);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+        s[rb][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k, qop[rb][ks], s[rb][kb], 0, 0, 0);
+    }
   }
   if (PREFETCH) {
 #pragma unroll
     for (int db = 0; db < NDB; ++db) vop1[db] = load_v(db, 1);
   }
-  float mx = -INFINITY;
+  bf16x8 pop[RB][2];
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
+  for (int rb = 0; rb < RB; ++rb) {
+    float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = k0 + key_of(kb, 4 * g + i);
-      const float v = (key >= me.first && key <= me.pos) ? s[kb][i] * scale : -INFINITY;
-      s[kb][i] = v;
-      mx = fmaxf(mx, v);
-    }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, FG_WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, FG_WAVE));
-  const float m_new = fmaxf(m, mx);
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-  const float alpha = __expf(m - m_use);                 // m = -inf: 0
-  float sum = 0.f;
-  bf16x8 pop[2];
+    for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-  for (int kb = 0; kb < 4; ++kb)
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + key_of(kb, 4 * g + i);
+        const float v = (key >= me[rb].first && key <= me[rb].pos) ? s[rb][kb][i] * scale : -INFINITY;
+        s[rb][kb][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, FG_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, FG_WAVE));
+    const float m_new = fmaxf(m[rb], mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+    const float alpha = __expf(m[rb] - m_use);             // m = -inf: 0
+    float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float p = __expf(s[kb][i] - m_use);
-      sum += p;
-      pop[kb >> 1][4 * (kb & 1) + i] = (__bf16)p;
-    }
-  l = l * alpha + sum;  // this lane's share of the row's sum; the groups are added at the end
-  m = m_new;
+    for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) {
-    o[db] *= alpha;
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? vop0[db] : load_v(db, 0), pop[0], o[db], 0, 0, 0);
+      for (int i = 0; i < 4; ++i) {
+        const float p = __expf(s[rb][kb][i] - m_use);
+        sum += p;
+        pop[rb][kb >> 1][4 * (kb & 1) + i] = (__bf16)p;
+      }
+    l[rb] = l[rb] * alpha + sum;  // this lane's share of the row's sum; the groups are added at the end
+    m[rb] = m_new;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[rb][db] *= alpha;
   }
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
-    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PREFETCH ? vop1[db] : load_v(db, 1), pop[1], o[db], 0, 0, 0);
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      const bf16x8 v = PREFETCH ? (ks == 0 ? vop0[db] : vop1[db]) : load_v(db, ks);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+        o[rb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pop[rb][ks], o[rb][db], 0, 0, 0);
+    }
 }
 
 // qrow is always a readable row; `valid` says whether it is this lane's
@@ -200,25 +212,25 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
 
   const int pos_last = it.pos0 + it.n_tok - 1;
   const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
-  ItemRows me{-1, 0};
+  ItemRows me[1] = {{-1, 0}};
   const bool my_row = r16 < it.n_tok * G;
   const int my_tok = my_row ? r16 / G : 0, my_head = my_row ? r16 % G : 0;
   if (my_row) {
-    me.pos = it.pos0 + my_tok;
-    me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
+    me[0].pos = it.pos0 + my_tok;
+    me[0].first = window > 0 && me[0].pos - window + 1 > 0 ? me[0].pos - window + 1 : 0;
   }
-  bf16x8 qop[NKS];
-  load_q(qop, q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
+  bf16x8 qop[1][NKS];
+  load_q(qop[0], q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
 
   const int t_lo = first_min / TILE, t_hi = pos_last / TILE;
   const int per_split = (t_hi - t_lo + 1 + n_splits - 1) / n_splits;
   const int t_begin = t_lo + split * per_split;
   const int t_end = min(t_hi + 1, t_begin + per_split);
 
-  float m = -INFINITY, l = 0.f;
-  f32x4 o[NDB];
+  float m_[1] = {-INFINITY}, l_[1] = {0.f};
+  f32x4 o_[1][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int db = 0; db < NDB; ++db) o_[0][db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const size_t head_elems = (size_t)page_size * HD;  // elements of one kv head in a page
   for (int t = t_begin + wave; t < t_end; t += 4) {
@@ -273,8 +285,10 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
       }
       return and_mask(v, vmask[ks]);
     };
-    attend_tile<true>(k0, me, qop, scale, m, l, o, load_k, load_v);
+    attend_tile<true, 1>(k0, me, qop, scale, m_, l_, o_, load_k, load_v);
   }
+  float m = m_[0], l = l_[0];
+  f32x4(&o)[NDB] = o_[0];
   l += __shfl_xor(l, 16, FG_WAVE);
   l += __shfl_xor(l, 32, FG_WAVE);
 
@@ -386,12 +400,15 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
 }
 
 // ------------------------------------------------------------------- tile
-// grid (n_items, n_kv), 256 threads: 4 waves of 16 rows; an item has at most
-// 64 / (H / KV) tokens.  The K and V tiles go through LDS in the order the
+// grid (n_items, n_kv), 256 threads: 4 waves of TILE_RB x 16 rows; an item has
+// at most TILE_ROWS / (H / KV) tokens.  The K and V tiles go through LDS in the order the
 // operands are read: K [4 key blocks][HD/8 chunks][16 keys][8], V [HD/16 dim
 // blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
+constexpr int TILE_RB = HD <= 128 ? 2 : 1;  // row blocks a wave holds (registers allow 2 up to head size 128)
+constexpr int TILE_ROWS = 64 * TILE_RB;     // query rows of an item
+
 template <bool PERM>
-__global__ __launch_bounds__(256) void attn_tile_kernel(
+__global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
@@ -408,28 +425,39 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int pos_last = it.pos0 + it.n_tok - 1;
   const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
 
-  const int row = wave * 16 + r16;
-  ItemRows me{-1, 0};
-  const bool my_row = row < it.n_tok * G;
-  const int my_tok = my_row ? row / G : 0, my_head = my_row ? row % G : 0;
-  if (my_row) {
-    me.pos = it.pos0 + my_tok;
-    me.first = window > 0 && me.pos - window + 1 > 0 ? me.pos - window + 1 : 0;
+  constexpr int RB = TILE_RB;
+  ItemRows me[RB];
+  bf16x8 qop[RB][NKS];
+  int w_hi = -1, w_lo = 0x7fffffff;  // the keys this wave's rows can see: tiles outside are skipped by the wave
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = (wave * RB + rb) * 16 + r16;
+    const bool my_row = row < it.n_tok * G;
+    const int my_tok = my_row ? row / G : 0, my_head = my_row ? row % G : 0;
+    me[rb] = ItemRows{-1, 0};
+    if (my_row) {
+      me[rb].pos = it.pos0 + my_tok;
+      me[rb].first = window > 0 && me[rb].pos - window + 1 > 0 ? me[rb].pos - window + 1 : 0;
+      w_hi = max(w_hi, me[rb].pos);
+      w_lo = min(w_lo, me[rb].first);
+    }
+    load_q(qop[rb], q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
   }
-  bf16x8 qop[NKS];
-  load_q(qop, q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
-  // the keys this wave's rows can see: tiles outside are skipped by the wave
-  int w_hi = me.pos, w_lo = me.pos < 0 ? 0x7fffffff : me.first;
 #pragma unroll
   for (int msk = 1; msk < 16; msk <<= 1) {
     w_hi = max(w_hi, __shfl_xor(w_hi, msk, FG_WAVE));
     w_lo = min(w_lo, __shfl_xor(w_lo, msk, FG_WAVE));
   }
 
-  float m = -INFINITY, l = 0.f;
-  f32x4 o[NDB];
+  float m[RB], l[RB];
+  f32x4 o[RB][NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb) {
+    m[rb] = -INFINITY;
+    l[rb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[rb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const size_t head_elems = (size_t)page_size * HD;
   constexpr int KCH = HD / 8;                  // 16-byte chunks in a key
@@ -501,19 +529,24 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
     auto load_v = [&](int db, int ks) -> bf16x8 {
       return *(const bf16x8*)(v_s + ((db * 8 + 4 * ks + g) * 16 + r16) * 8);
     };
-    attend_tile<false>(k0, me, qop, scale, m, l, o, load_k, load_v);
+    attend_tile<false, RB>(k0, me, qop, scale, m, l, o, load_k, load_v);
   }
-  l += __shfl_xor(l, 16, FG_WAVE);
-  l += __shfl_xor(l, 32, FG_WAVE);
-  if (row < it.n_tok * G) {
-    bf16_t* orow = out + (size_t)(it.tok0 + row / G) * out_stride + (size_t)(kvh * G + row % G) * HD;
-    const float inv = 1.f / l;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      bf16x4 v;
+  for (int rb = 0; rb < RB; ++rb) {
+    float lsum = l[rb];
+    lsum += __shfl_xor(lsum, 16, FG_WAVE);
+    lsum += __shfl_xor(lsum, 32, FG_WAVE);
+    const int row = (wave * RB + rb) * 16 + r16;
+    if (row < it.n_tok * G) {
+      bf16_t* orow = out + (size_t)(it.tok0 + row / G) * out_stride + (size_t)(kvh * G + row % G) * HD;
+      const float inv = 1.f / lsum;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[db][i] * inv);
-      *(bf16x4*)(orow + 16 * db + 4 * g) = v;
+      for (int db = 0; db < NDB; ++db) {
+        bf16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[rb][db][i] * inv);
+        *(bf16x4*)(orow + 16 * db + 4 * g) = v;
+      }
     }
   }
 }
@@ -523,7 +556,7 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
                             int n_items, int n_heads, int n_kv, int hd, int page_size, float scale, int window,
                             hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
-  if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 64 || page_size < 8 || page_size % 8 ||
+  if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > TILE_ROWS || page_size < 8 || page_size % 8 ||
       n_kv > 65535 || window < 0 || q_stride % 8 || out_stride % 4)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                        \
@@ -536,3 +569,5 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
 }
 
 extern "C" int fg_attn_head_dim() { return HD; }
+// query rows (tokens x heads of a kv head's group) of one item of fg_attn_tile
+extern "C" int fg_attn_tile_rows() { return TILE_ROWS; }

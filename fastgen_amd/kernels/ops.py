@@ -240,24 +240,30 @@ MFMA_MAX_HEAD_DIM = 256
 _SPLIT_TARGET_BLOCKS = 1024  # workgroups wanted in flight for the decode kernel (4 per CU)
 
 
-def attention_items(q_lens, q_start, n_cached, group_size: int):
+def attention_tile_rows(head_dim: int) -> int:
+    """Query rows of one item of the tile kernel for this head size."""
+    return int(_lib.load(f"attention_mfma@{head_dim}").fg_attn_tile_rows())
+
+
+def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int = 64):
     """Cut the step's sequences into items for the MFMA kernels.
 
     Returns two int32 arrays ``[n, 4]`` of (sequence, first flat token, tokens,
     position of the first token): items of at most 16 rows for the split
-    kernel (decoded tokens and very short portions) and items of at most 64
-    rows for the tile kernel.
+    kernel (decoded tokens and very short portions) and items of at most
+    ``tile_rows`` rows for the tile kernel, those with the most keys first.
     """
     import numpy as np
 
     small, big = [], []
-    per_tile = max(1, 64 // group_size)
+    per_tile = max(1, tile_rows // group_size)
     for b, n in enumerate(q_lens):
         n, s, c = int(n), int(q_start[b]), int(n_cached[b])
         if n * group_size <= 16:
             small.append((b, s, n, c))
         else:
             big.extend((b, s + i, min(per_tile, n - i), c + i) for i in range(0, n, per_tile))
+    big.sort(key=lambda it: -(it[3] + it[2]))  # the longest key ranges start first
     as_arr = lambda x: np.asarray(x, dtype=np.int32).reshape(-1, 4)
     return as_arr(small), as_arr(big)
 
@@ -304,7 +310,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                 n_splits, n_heads, n_kv, hd, page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
             _check(st, "attn_split")
     if big_items is not None and big_items.numel():
-        _need(G <= 64, "the tile kernel takes at most 64 query heads per kv head")
+        _need(G <= attention_tile_rows(hd), "too many query heads per kv head for the tile kernel")
         _i32(big_items, "big_items")
         _need(big_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
         st = lib.fg_attn_tile(
@@ -339,7 +345,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
             # already (and are refreshed with it when the step is a replayed graph)
             plan = (ctx.seq_records, None, ctx.n_seqs)
         else:
-            small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G)
+            small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, attention_tile_rows(hd))
             both = torch.from_numpy(np.concatenate([small, big]).reshape(-1)).to(q.device)
             plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small))
         ctx.scratch[("attention_items", G)] = plan

@@ -413,7 +413,8 @@ def _run_mfma(ops, case, seqs, H, KV, window=0, n_splits=1):
 
     q_lens = [b for _, b in seqs]
     q_start = np.concatenate([[0], np.cumsum(q_lens)])
-    small, big = ops.attention_items(q_lens, q_start, [a for a, _ in seqs], H // KV)
+    small, big = ops.attention_items(q_lens, q_start, [a for a, _ in seqs], H // KV,
+                                     ops.attention_tile_rows(case["kp"].shape[3]))
     dev = lambda a: torch.from_numpy(a.reshape(-1)).to(DEV) if a.size else None
     out = torch.full_like(case["q"], float("nan"))
     ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], dev(small), dev(big), H,
