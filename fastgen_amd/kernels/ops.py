@@ -237,7 +237,13 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
 
 
 MFMA_MAX_HEAD_DIM = 256
-_SPLIT_TARGET_BLOCKS = 1024  # workgroups wanted in flight for the decode kernel (4 per CU)
+import os as _os
+
+# Workgroups wanted for the decode attention kernel: one per CU measured best (256 CUs; 128 to 2048
+# tried at batch 1, 8 and 64).  The splits' partial results are merged by a second kernel: merging
+# them in the split that finishes last needs device-scope fences, which on a GPU of several
+# dies cost more than the launch they save (measured).
+_SPLIT_TARGET_BLOCKS = int(_os.environ.get("FG_SPLIT_TARGET", 256))
 
 
 def attention_tile_rows(head_dim: int) -> int:
