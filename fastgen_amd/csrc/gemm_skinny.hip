@@ -173,6 +173,89 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
   }
 }
 
+// More rows of x (17..64): a workgroup owns 64 rows of W, one 16-row block a
+// wave over the whole k range of the workgroup, so nothing is reduced across
+// waves; the workgroup's slice of x for the next 8 k steps (MB*16 rows x 256)
+// goes through LDS once for all four waves.  blockIdx.y cuts K: split s adds
+// rows k in [s*k_per_split, ...) and stores its partial sums at y + s *
+// part_stride (fp32); the consumer adds the partials in split order.
+template <int MB, int EPI, class TY>
+__global__ __launch_bounds__(256) void gemm_skinny64_kernel(
+    const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
+    int ldy, size_t part_stride, int M, int N, int K, int k_per_split) {
+  constexpr int U = 8;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][4 * U * MB * 16 * 8];  // [buffer][k chunk][row][8]
+  const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const int k_begin = min(K, (int)blockIdx.y * k_per_split), k_end = min(K, k_begin + k_per_split);
+  f32x4 acc[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // copying x: 32 chunks a row and iteration; thread t copies chunk t % 32 of rows t / 32 + 8 j
+  const int c_chunk = threadIdx.x & 31, c_row = threadIdx.x >> 5;
+  constexpr int XL = MB * 2;  // loads a thread issues for the x slice
+  // The loads of the next 8 k steps (W and the x slice) are in flight while the current ones are
+  // multiplied: they are issued right after the barrier that publishes the current x slice.
+  bf16x8 a_next[U], xv[XL];
+  auto fetch = [&](int kk) {
+#pragma unroll
+    for (int j = 0; j < XL; ++j) {
+      const int row = min(c_row + 8 * j, M - 1), k = kk + 8 * c_chunk;
+      xv[j] = *(const bf16x8*)(x + (size_t)row * ldx + (k < k_end ? k : k_begin));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = kk + 32 * u + 8 * g;
+      const bool in = k < k_end;
+      const bf16x8 av = *(const bf16x8*)(wrow + (in ? k : k_begin));
+      a_next[u] = in ? av : gs_zero8();
+    }
+  };
+  if (k_begin < k_end) fetch(k_begin);
+  int buf = 0;
+  for (int kk = k_begin; kk < k_end; kk += 32 * U, buf ^= 1) {
+    bf16_t* my = xs[buf];
+#pragma unroll
+    for (int j = 0; j < XL; ++j) *(bf16x8*)(my + (c_chunk * (MB * 16) + c_row + 8 * j) * 8) = xv[j];
+    bf16x8 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) a[u] = a_next[u];
+    __syncthreads();  // this buffer is complete; the other one may still be read by slower waves
+    if (kk + 32 * U < k_end) fetch(kk + 32 * U);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const bf16x8 b = *(const bf16x8*)(my + ((4 * u + g) * (MB * 16) + 16 * mb + r16) * 8);
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[mb], 0, 0, 0);
+      }
+  }
+  // acc[mb][i] = C[n = n0 + 4g + i][m = 16 mb + r16]
+  TY* yp = y + (size_t)blockIdx.y * part_stride;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int m = 16 * mb + r16;
+    if (EPI == EPI_STORE) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g + i;
+        if (m < M && n < N) yp[(size_t)m * ldy + n] = from_f<TY>(acc[mb][i]);
+      }
+    } else {
+      // lane groups 0,1 hold gate rows 4g+i of 8 channels, groups 2,3 the up rows of the same channels
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float other = __shfl_xor(acc[mb][i], 32, FG_WAVE);
+        const float gate = acc[mb][i], up = other;
+        const int col = n0 / 2 + 4 * g + i;
+        if (g < 2 && m < M && n0 + 8 + 4 * g + i < N) yp[(size_t)m * ldy + col] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
+      }
+    }
+  }
+}
+
 template <int MB, int EPI, class TY>
 static void launch_skinny(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
                           int K, hipStream_t stream) {
@@ -222,5 +305,39 @@ extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, vo
   else if (mb == 3) GO(3);
   else GO(4);
 #undef GO
+  return fg_launch_status();
+}
+
+// x [M, K] bf16 with 16 < M <= 64 (fewer rows work too).  k_splits > 1: y is fp32 [k_splits, M, N]
+// (part_stride elements apart), partial sums over K to be added by the consumer in split order;
+// only with epilogue 0.
+extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, void* y, int ldy,
+                                long long part_stride, int k_splits, int M, int N, int K, int out_dtype,
+                                int epilogue, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return FG_OK;
+  if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535)
+    return FG_ERR_ARG;
+  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
+  if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
+  if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
+  const int k_per_split = ((K + k_splits * 256 - 1) / (k_splits * 256)) * 256;
+  const dim3 grid((N + 63) / 64, k_splits);
+  const int mb = (M + 15) / 16;
+#define GO64(MB, EPI, TY)                                                                              \
+  gemm_skinny64_kernel<MB, EPI, TY><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
+                                                              ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split)
+#define PICK(MB)                                                                   \
+  do {                                                                             \
+    if (epilogue == EPI_SILU_MUL) GO64(MB, EPI_SILU_MUL, bf16_t);                  \
+    else if (out_dtype == FG_BF16) GO64(MB, EPI_STORE, bf16_t);                    \
+    else if (out_dtype == FG_F32) GO64(MB, EPI_STORE, float);                      \
+    else return FG_ERR_ARG;                                                        \
+  } while (0)
+  if (mb == 1) PICK(1);
+  else if (mb == 2) PICK(2);
+  else if (mb == 3) PICK(3);
+  else PICK(4);
+#undef PICK
+#undef GO64
   return fg_launch_status();
 }

@@ -42,22 +42,26 @@ extern "C" int fg_embed(const void* table, int table_dtype, const int* tokens, f
 // the sum is written back to h, so the residual stream is updated in the pass
 // that reads it for the norm; a gathered call leaves h as it is (rows may
 // name a row twice).
+// What is added to h is either `delta` (rows of the activation dtype) or the sum, in order, of
+// `n_parts` fp32 partial results `parts[p]` (a matrix product whose k range was cut).
 template <class TA, class TW>
 __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_kernel(
-    float* __restrict__ h, const TA* __restrict__ delta, const TW* __restrict__ w,
-    TA* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
+    float* __restrict__ h, const TA* __restrict__ delta, const float* __restrict__ parts, int n_parts,
+    size_t part_stride, const TW* __restrict__ w, TA* __restrict__ out, const int* __restrict__ rows, int dim,
+    float eps) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   float* hrow = h + src * dim;
   const TA* drow = delta ? delta + src * dim : nullptr;
+  const bool adds = drow || parts;
   float ss = 0.f;
   for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
     float v = hrow[i];
-    if (drow) {
-      v += to_f<TA>(drow[i]);
-      if (!rows) hrow[i] = v;
-    }
+    if (drow) v += to_f<TA>(drow[i]);
+    if (parts)
+      for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + src * dim + i];
+    if (adds && !rows) hrow[i] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
@@ -66,7 +70,11 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_kernel(
   for (int i = threadIdx.x; i < dim; i += ROWS_THREADS) {
     // each thread re-reads only what it wrote itself above
     float v = hrow[i];
-    if (drow && rows) v += to_f<TA>(drow[i]);
+    if (rows) {
+      if (drow) v += to_f<TA>(drow[i]);
+      if (parts)
+        for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + src * dim + i];
+    }
     orow[i] = from_f<TA>(v * rstd * to_f<TW>(w[i]));
   }
 }
@@ -76,8 +84,9 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_kernel(
 // once.  For dim % 8 == 0 and dim <= 2048 * NIT.
 template <class TA, class TW, int NIT>
 __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
-    float* __restrict__ h, const TA* __restrict__ delta, const TW* __restrict__ w,
-    TA* __restrict__ out, const int* __restrict__ rows, int dim, float eps) {
+    float* __restrict__ h, const TA* __restrict__ delta, const float* __restrict__ parts, int n_parts,
+    size_t part_stride, const TW* __restrict__ w, TA* __restrict__ out, const int* __restrict__ rows, int dim,
+    float eps) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -89,15 +98,30 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
     const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
     if (e < dim) load8<float>(hrow + e, v[it]);
   }
-  if (drow) {
+  if (drow || parts) {
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
       if (e < dim) {
         float d[8];
-        load8<TA>(drow + e, d);
+        if (drow) {
+          load8<TA>(drow + e, d);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[it][i] += d[i];
+          for (int i = 0; i < 8; ++i) v[it][i] += d[i];
+        }
+        if (parts) {
+          // eight partial results at a time, all loads issued before the first is added
+          for (int p0 = 0; p0 < n_parts; p0 += 8) {
+            float dp[8][8];
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+              load8<float>(parts + (size_t)min(p0 + p, n_parts - 1) * part_stride + src * dim + e, dp[p]);
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+#pragma unroll
+              for (int i = 0; i < 8; ++i) v[it][i] += p0 + p < n_parts ? dp[p][i] : 0.f;
+          }
+        }
         if (!rows) store8<float>(hrow + e, v[it]);
       }
     }
@@ -128,26 +152,28 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
 }
 
 template <class TA, class TW>
-static void launch_add_rmsnorm(float* h, const void* delta, const void* w, void* out, const int* rows,
-                               int n_rows, int dim, float eps, hipStream_t stream) {
+static void launch_add_rmsnorm(float* h, const void* delta, const float* parts, int n_parts, size_t part_stride,
+                               const void* w, void* out, const int* rows, int n_rows, int dim, float eps,
+                               hipStream_t stream) {
 #define VEC(NIT)                                                                              \
   add_rmsnorm_vec_kernel<TA, TW, NIT><<<n_rows, ROWS_THREADS, 0, stream>>>(                   \
-      h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps)
+      h, (const TA*)delta, parts, n_parts, part_stride, (const TW*)w, (TA*)out, rows, dim, eps)
   if (dim % 8 == 0 && dim <= 2048) VEC(1);
   else if (dim % 8 == 0 && dim <= 4096) VEC(2);
   else if (dim % 8 == 0 && dim <= 8192) VEC(4);
   else
     add_rmsnorm_kernel<TA, TW><<<n_rows, ROWS_THREADS, 0, stream>>>(
-        h, (const TA*)delta, (const TW*)w, (TA*)out, rows, dim, eps);
+        h, (const TA*)delta, parts, n_parts, part_stride, (const TW*)w, (TA*)out, rows, dim, eps);
 #undef VEC
 }
 
-extern "C" int fg_add_rmsnorm(float* h, const void* delta, const void* w, void* out,
-                              const int* rows, int n_rows, int dim, float eps, int act_dtype,
-                              int w_dtype, hipStream_t stream) {
+extern "C" int fg_add_rmsnorm(float* h, const void* delta, const float* parts, int n_parts,
+                              long long part_stride, const void* w, void* out, const int* rows, int n_rows,
+                              int dim, float eps, int act_dtype, int w_dtype, hipStream_t stream) {
   if (n_rows <= 0) return FG_OK;
-  if (dim <= 0) return FG_ERR_ARG;
-#define LAUNCH(TA, TW) launch_add_rmsnorm<TA, TW>(h, delta, w, out, rows, n_rows, dim, eps, stream)
+  if (dim <= 0 || (parts && n_parts < 1)) return FG_ERR_ARG;
+#define LAUNCH(TA, TW) \
+  launch_add_rmsnorm<TA, TW>(h, delta, parts, n_parts, (size_t)part_stride, w, out, rows, n_rows, dim, eps, stream)
   if (act_dtype == FG_F32 && w_dtype == FG_F32) LAUNCH(float, float);
   else if (act_dtype == FG_BF16 && w_dtype == FG_BF16) LAUNCH(bf16_t, bf16_t);
   else if (act_dtype == FG_BF16 && w_dtype == FG_F32) LAUNCH(bf16_t, float);

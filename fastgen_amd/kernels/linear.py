@@ -35,18 +35,38 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
         raise
 
 
-# up to this many rows the weight-streaming kernel is faster than the library's product
-SKINNY_ROWS = 16
+# up to this many rows the weight-streaming kernels are used (more: the library's product)
+SKINNY_ROWS = 16  # one 16-row block of x, 16 output columns a workgroup
+WIDE_ROWS = 64    # up to four blocks of x, 64 output columns a workgroup
 
 
-def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Few rows (decode): the engine's own weight-streaming kernel takes the product."""
-    return (x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0
+def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
             and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Few rows (decode): the engine's own weight-streaming kernel takes the product."""
+    return x.shape[0] <= SKINNY_ROWS and _aligned(x, w)
+
+
+def wide_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Up to 64 rows: the engine's kernel where it beats the library (fused epilogue, or k splits)."""
+    return x.shape[0] <= WIDE_ROWS and _aligned(x, w)
+
+
+def k_splits_for(n_out: int, k: int) -> int:
+    """Splits of the k range that give the wide kernel about two workgroups per CU."""
+    blocks = -(-n_out // 64)
+    return max(1, min(8, 512 // blocks, k // 512))
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           partials_ok: bool = False) -> torch.Tensor:
+    """``x @ w.T``.  With ``partials_ok`` the result may come as fp32 ``[S, M, N]``
+    partial sums whose sum over ``S`` is the product (the caller hands it to a
+    norm, which adds them in order)."""
     if not x.is_cuda:
         raise ops.KernelArgumentError("fastgen_amd runs on the GPU only; got a tensor on " + str(x.device))
     out_dtype = out_dtype or x.dtype
@@ -56,8 +76,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return ops.gemm_nt(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
+    if partials_ok and x.shape[0] > 2 and wide_ok(x, w) and w.shape[0] <= 8192:
+        splits = k_splits_for(w.shape[0], w.shape[1])
+        if splits > 1:
+            return ops.gemm_skinny(x, w, k_splits=splits, wide=True)
     if skinny_ok(x, w):
-        return ops.gemm_skinny(x, w, out_dtype)
+        return ops.gemm_skinny(x, w, out_dtype, wide=False)
     if out_dtype == torch.bfloat16:
         return torch.nn.functional.linear(x, w)
     y = _library_mm_f32_out(x, w)

@@ -85,8 +85,10 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``h += delta`` (fp32 residual stream), ``out = rmsnorm(h) * weight``.
 
-    With ``rows`` only those rows of ``h`` are normed, into consecutive rows
-    of ``out``, and ``h`` is left unchanged.  Norm as in
+    ``delta`` is ``[T, dim]`` of ``out``'s dtype, or fp32 ``[S, T, dim]``: partial
+    sums of a matrix product whose k range was cut, added in order.  With
+    ``rows`` only those rows of ``h`` are normed, into consecutive rows of
+    ``out``, and ``h`` is left unchanged.  Norm as in
     ``fastgen/kernels/rmsnorm.py:33-60``.
     """
     _gpu(h, delta, weight, out, rows)
@@ -97,12 +99,17 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _i32(rows, "rows")
     _need(weight.shape == (dim,) and weight.is_contiguous(), "weight must be [dim]")
     _need(out.is_contiguous() and out.shape == (n_rows, dim), "out must be contiguous [rows, dim]")
-    if delta is not None:
+    parts, n_parts, part_stride = None, 0, 0
+    if delta is not None and delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and delta.shape[1:] == h.shape and delta.stride(2) == 1
+              and delta.stride(1) == dim, "partial sums must be float32 [S, T, dim] with contiguous rows")
+        parts, n_parts, part_stride, delta = delta, delta.shape[0], delta.stride(0), None
+    elif delta is not None:
         _need(delta.shape == h.shape and delta.is_contiguous() and delta.dtype == out.dtype,
               "delta must be contiguous, shaped like h, of out's dtype")
     st = _lib.load("rows").fg_add_rmsnorm(
-        _ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), n_rows, dim, ctypes.c_float(eps),
-        _code(out), _code(weight), _stream(out))
+        _ptr(h), _ptr(delta), _ptr(parts), n_parts, ctypes.c_longlong(part_stride), _ptr(weight), _ptr(out),
+        _ptr(rows), n_rows, dim, ctypes.c_float(eps), _code(out), _code(weight), _stream(out))
     _check(st, "add_rmsnorm")
     return out
 
@@ -391,11 +398,15 @@ SKINNY_MAX_ROWS = 64
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-                silu_mul_epilogue: bool = False) -> torch.Tensor:
+                silu_mul_epilogue: bool = False, k_splits: int = 1, wide: Optional[bool] = None) -> torch.Tensor:
     """``x @ w.T`` for at most 64 rows of bf16 ``x`` on the matrix cores, built to
     stream ``w [N, K]`` once.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
     ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
-    ``[M, N/2]``."""
+    ``[M, N/2]``.  With ``k_splits > 1`` the k range is cut over workgroups and the
+    result is fp32 ``[k_splits, M, N]`` partial sums (for few output columns,
+    where one workgroup per 64 columns would leave most of the GPU idle).
+    ``wide`` picks the kernel for 17..64 rows (64 columns a workgroup, x shared
+    through LDS); default: by the number of rows."""
     _gpu(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16 operands")
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
@@ -407,10 +418,21 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     out_dtype = out_dtype or torch.bfloat16
     if silu_mul_epilogue:
         _need(N % 16 == 0 and out_dtype == torch.bfloat16, "the gate/up epilogue needs N % 16 == 0 and bf16 output")
-    y = torch.empty((M, N // 2 if silu_mul_epilogue else N), dtype=out_dtype, device=x.device)
-    st = _lib.load("gemm_skinny").fg_gemm_skinny(
-        _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, _code(y),
-        1 if silu_mul_epilogue else 0, _stream(x))
+    wide = (M > 16 or k_splits > 1) if wide is None else wide
+    _need(k_splits >= 1 and (k_splits == 1 or (wide and not silu_mul_epilogue)), "k_splits needs the wide kernel")
+    if k_splits > 1:
+        out_dtype = torch.float32
+    cols = N // 2 if silu_mul_epilogue else N
+    y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
+    lib = _lib.load("gemm_skinny")
+    if wide:
+        st = lib.fg_gemm_skinny64(
+            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
+            K, _code(y), 1 if silu_mul_epilogue else 0, _stream(x))
+    else:
+        st = lib.fg_gemm_skinny(
+            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, _code(y),
+            1 if silu_mul_epilogue else 0, _stream(x))
     _check(st, "gemm_skinny")
     return y
 

@@ -29,6 +29,11 @@ class Attention(Mixer):
         self.window: Optional[int] = o.get("window") or None
         if self.n_heads % self.n_kv_heads:
             raise ValueError(f"n_heads={self.n_heads} is not a multiple of n_kv_heads={self.n_kv_heads}")
+        if self.head_dim % 8 or self.head_dim > 512:
+            raise ValueError(
+                f"{self.prefix}: head size {self.head_dim} is not supported: the cache and the attention"
+                " kernels work in chunks of 8 head dimensions, up to 512"
+            )
         self.position = build_part("position", o["position"])
         self.wqkv: Optional[torch.Tensor] = None
         self.wo: Optional[torch.Tensor] = None
@@ -76,7 +81,7 @@ class Attention(Mixer):
         out = torch.empty((x.shape[0], q_width), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,
                             self.window or 0)
-        return linear(out, self.wo)
+        return linear(out, self.wo, partials_ok=True)
 
 
 register_part("mixer", "attention", Attention)

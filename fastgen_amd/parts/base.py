@@ -97,8 +97,10 @@ class Mixer(Part):
 
     ``forward(x, ctx, store)`` gets the normed rows ``[T, dim]`` of the step,
     the step's ragged description and its storage, and returns ``[T, dim]``
-    rows in the same dtype to be added to the residual stream.  What one step
-    writes to the storage is what the next step of the same request reads.
+    rows in the same dtype to be added to the residual stream (or fp32
+    ``[S, T, dim]`` partial sums whose sum is that; the norm adds them).  What
+    one step writes to the storage is what the next step of the same request
+    reads.
     """
 
     def paged_need(self) -> Optional[PagedNeed]:
@@ -123,7 +125,8 @@ class Norm(Part):
 
     ``forward(h, delta, rows=None)`` adds ``delta`` (or nothing) to ``h`` in
     place and returns the normed rows in ``dtype``; with ``rows`` only those
-    rows are returned and ``h`` is left as it was.
+    rows are returned and ``h`` is left as it was.  ``delta`` is ``[T, dim]`` in
+    ``dtype`` or fp32 ``[S, T, dim]`` partial sums to be added in order.
     """
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor], dtype: torch.dtype,

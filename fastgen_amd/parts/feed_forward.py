@@ -11,7 +11,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear, skinny_ok
+from ..kernels.linear import linear, wide_ok
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
@@ -38,11 +38,11 @@ class SwiGLU(FeedForward):
         self.w_down = place(tensors[self._name("down_proj.weight")], MATRIX, dtype, device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if skinny_ok(x, self.w_gate_up):
+        if wide_ok(x, self.w_gate_up):
             act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True)
         else:
             act = ops.silu_mul(linear(x, self.w_gate_up))
-        return linear(act, self.w_down)
+        return linear(act, self.w_down, partials_ok=True)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -171,6 +171,13 @@ def test_random_weights_folder(tmp_path):
         read_config_json(tmp_path)
 
 
+def test_sizes_the_kernels_cannot_take_are_refused_when_the_model_is_built():
+    arch = get_architecture(TINY_A)
+    bad_head = dict(TINY_A, hidden_size=80, num_attention_heads=4, num_key_value_heads=2)  # head size 20
+    with pytest.raises(ValueError, match="head size 20 is not supported"):
+        build_parts(arch.layout(arch.parse(bad_head)))
+
+
 def test_dtype_policy():
     from fastgen_amd.parts import MATRIX, VECTOR, TABLE_INT, place
 

@@ -15,6 +15,10 @@ import traces
 from helpers import assert_close, make_runner, plain_logits, run_trace, save_model_folder
 from plain_llama import TINY_A, TINY_B, TINY_C, plain_forward, plain_random_weights
 
+# one kv head for 32 query heads (wider than the MFMA kernels' groups), head size 24 (not a multiple of 16)
+TINY_D = dict(TINY_A, hidden_size=32 * 24, num_attention_heads=32, num_key_value_heads=1, intermediate_size=136,
+              num_hidden_layers=1, vocab_size=131, tie_word_embeddings=False)
+
 pytestmark = pytest.mark.gpu
 
 REPO = Path(__file__).resolve().parent.parent
@@ -24,6 +28,7 @@ CASES = {
     "A": (TINY_A, 0, 16, {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 1}),
     "B": (TINY_B, 1, 32, {"a": 1, "b": 12, "c": 40, "d": 90, "e": 150, "f": 129}),
     "C": (TINY_C, 2, 64, {"a": 70, "b": 200, "c": 2, "d": 64, "e": 131}),
+    "D": (TINY_D, 3, 8, {"a": 9, "b": 70, "c": 33, "d": 3, "e": 40}),
 }
 
 

@@ -302,6 +302,43 @@ def test_gemm_skinny(ops, M, N, K, odtype):
     assert err < (1e-5 if odtype == torch.float32 else 6e-3), float(err)
 
 
+@pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("N,K,S", [(515, 240, 1), (4096, 4096, 4), (4096, 14336, 8), (100, 264, 3), (6144, 64, 1)])
+def test_gemm_skinny_wide_and_k_splits(ops, M, N, K, S):
+    torch.manual_seed(17)
+    x, w = torch.randn(M, K).bfloat16(), (torch.randn(N, K) * 0.1).bfloat16()
+    got = ops.gemm_skinny(x.to(DEV), w.to(DEV), k_splits=S, wide=True)
+    want = x.double() @ w.double().T
+    if S > 1:
+        assert got.dtype == torch.float32 and got.shape == (S, M, N)
+        total = got.cpu().double().sum(0)
+        assert (total - want).abs().max() / want.abs().max() < 1e-5
+        # the norm that follows adds the partial sums itself
+        h = torch.randn(M, N)
+        wn = 1 + 0.1 * torch.randn(N)
+        hd, out = h.to(DEV), torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.add_rmsnorm(hd, got, wn.to(DEV), 1e-5, out)
+        hs = h + got.cpu().sum(0)
+        assert torch.allclose(hd.cpu(), hs, atol=1e-4 * float(hs.abs().max()))
+        ref = (hs * torch.rsqrt((hs * hs).mean(-1, keepdim=True) + 1e-5) * wn).bfloat16()
+        assert torch.allclose(out.cpu().float(), ref.float(), atol=2e-2, rtol=2e-2)
+    else:
+        assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+        assert (got.cpu().double() - want).abs().max() / want.abs().max() < 6e-3
+
+
+@pytest.mark.parametrize("M", [17, 64])
+def test_gemm_skinny_wide_gate_up(ops, M):
+    torch.manual_seed(18)
+    F, K = 1000, 328
+    x = torch.randn(M, K).bfloat16()
+    wg, wu = (torch.randn(F, K) * 0.05).bfloat16(), (torch.randn(F, K) * 0.05).bfloat16()
+    got = ops.gemm_skinny(x.to(DEV), ops.interleave_gate_up(wg, wu).contiguous().to(DEV), silu_mul_epilogue=True).cpu()
+    g, u = x.float() @ wg.float().T, x.float() @ wu.float().T
+    want = g * torch.sigmoid(g) * u
+    assert got.shape == (M, F) and (got.float() - want).abs().max() <= 1e-2 * want.abs().max() + 1e-3
+
+
 def test_gemm_skinny_takes_views_and_refuses_the_rest(ops):
     from fastgen_amd.kernels import KernelArgumentError
 
