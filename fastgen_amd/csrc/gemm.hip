@@ -1,9 +1,11 @@
 // y = x W^T with W stored [out, in] row-major (fastgen/forward.py:433-440,
 // 470, 488-496, 513: F.linear).  This is the engine's own matrix product for
 // the true 32-bit path: plain fp32 fused multiply-adds, no matrix-core mode of
-// reduced precision.  Every output element is one dot product summed over k
-// in ascending order by one thread, so a row's result does not depend on how
-// many other rows the call holds.  It also takes bf16 operands (fp32
+// reduced precision.  Every output element is one dot product summed by one
+// thread in an order fixed by K alone (16 products into a partial sum, 16
+// partial sums into a second one, those into the total: rounding grows with
+// K/256 + 32, not with K), so a row's result does not depend on how many other
+// rows the call holds.  It also takes bf16 operands (fp32
 // accumulate) so that any shape has a product when the tuned ones refuse it.
 #include "common.h"
 
@@ -22,11 +24,12 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_nt_kernel(
   const int tid = threadIdx.x;
   const int m0 = blockIdx.y * GT_M, n0 = blockIdx.x * GT_N;
   const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
-  float acc[4][4];
+  float acc[4][4], mid[4][4];  // total; sum of up to 16 tiles' partial sums
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = mid[i][j] = 0.f;
+  int tiles_in_mid = 0;
 
   // each thread loads 4 elements of each tile: row = tid / 4, k = (tid % 4) * 4 ..
   const int lr = tid / 4, lk = (tid % 4) * 4;
@@ -39,6 +42,11 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_nt_kernel(
       ws[lk + e][lr] = (n < N && k < K) ? to_f<TW>(w[(size_t)n * ldw + k]) : 0.f;
     }
     __syncthreads();
+    float part[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int k = 0; k < GT_K; ++k) {
       float a[4], b[4];
@@ -49,10 +57,26 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_nt_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+    const bool fold = ++tiles_in_mid == 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mid[i][j] += part[i][j];
+        if (fold) {
+          acc[i][j] += mid[i][j];
+          mid[i][j] = 0.f;
+        }
+      }
+    if (fold) tiles_in_mid = 0;
     __syncthreads();
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] += mid[i][j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + tm + i;

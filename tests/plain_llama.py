@@ -15,6 +15,12 @@ from typing import Dict, Mapping, Optional
 import torch
 
 
+def _up(x: torch.Tensor) -> torch.Tensor:
+    """To the precision of the fp32 islands: float32, or float64 when the whole
+    run is in float64 (used to judge float32 runs of wide layers)."""
+    return x if x.dtype == torch.float64 else x.float()
+
+
 def plain_rope_frequencies(head_dim: int, theta: float, scaling: Optional[Mapping] = None) -> torch.Tensor:
     """fastgen/forward.py:609-635.  ``scaling`` holds the config.json keys
     ``factor``, ``low_freq_factor``, ``high_freq_factor``,
@@ -45,8 +51,8 @@ def plain_rope_interleaved(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tens
     x ``[T, heads, hd]``; pair (x[2i], x[2i+1]) rotated by pos * freqs[i]."""
     angles = pos.to(torch.float32)[:, None] * freqs[None, :]  # [T, hd/2]
     cos, sin = torch.cos(angles)[:, None, :], torch.sin(angles)[:, None, :]
-    re, im = x[..., 0::2].float(), x[..., 1::2].float()
-    out = torch.empty_like(x, dtype=torch.float32)
+    re, im = _up(x[..., 0::2]), _up(x[..., 1::2])
+    out = torch.empty_like(x, dtype=re.dtype)
     out[..., 0::2] = re * cos - im * sin
     out[..., 1::2] = im * cos + re * sin
     return out.to(x.dtype)
@@ -62,9 +68,9 @@ def plain_rope_shuffle(w: torch.Tensor, n_heads: int) -> torch.Tensor:
 
 def plain_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
     """fastgen/kernels/rmsnorm.py:33-60: fp32 mean of squares, a * rstd * w."""
-    xf = x.float()
+    xf = _up(x)
     rstd = torch.rsqrt((xf * xf).sum(-1, keepdim=True) / x.shape[-1] + eps)
-    return (xf * rstd * w.float()).to(x.dtype)
+    return (xf * rstd * _up(w)).to(x.dtype)
 
 
 def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: Optional[int] = None) -> torch.Tensor:
@@ -81,8 +87,8 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: O
     if window:
         mask &= idx[None, :] > idx[:, None] - window
     for h in range(H):
-        kh, vh = k[:, h // G].float(), v[:, h // G].float()
-        s = (q[:, h].float() @ kh.T) * scale
+        kh, vh = _up(k[:, h // G]), _up(v[:, h // G])
+        s = (_up(q[:, h]) @ kh.T) * scale
         s = s.masked_fill(~mask, float("-inf"))
         p = torch.softmax(s, dim=-1)
         out[:, h] = (p @ vh).to(q.dtype)
@@ -133,7 +139,7 @@ def plain_forward(weights: Mapping[str, torch.Tensor], config: Mapping, tokens, 
                              W[p + "mlp.down_proj.weight"])  # forward.py:483-499
     h = plain_rmsnorm(h, W["model.norm.weight"], eps)  # forward.py:501
     head = W["model.embed_tokens.weight"] if config.get("tie_word_embeddings") else W["lm_head.weight"]
-    return (h @ head.T).float()  # forward.py:507-515
+    return _up(h @ head.T)  # forward.py:507-515
 
 
 def plain_greedy(weights, config, prompt, n_new: int, dtype=torch.float32):

@@ -1,0 +1,52 @@
+"""The layer sizes of the architecture's real family (Llama 3.1 8B: hidden
+4096, 32 heads over 8 kv heads of 128, feed-forward 14336, llama3 rope
+scaling), two layers and a smaller vocabulary so that the plain
+implementation stays fast: the kernels' production shapes under every way of
+cutting, in 32-bit and in bfloat16."""
+
+import pytest
+import torch
+
+import traces
+from helpers import assert_close, make_runner, plain_logits, run_trace, save_model_folder
+from plain_llama import plain_forward, plain_random_weights
+
+pytestmark = pytest.mark.gpu
+
+FAMILY = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=4096, intermediate_size=14336, num_hidden_layers=2,
+    num_attention_heads=32, num_key_value_heads=8, rms_norm_eps=1e-5, vocab_size=32003, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=False, max_position_embeddings=131072,
+)
+LENGTHS = {"a": 200, "b": 70, "c": 129, "d": 33}
+
+
+@pytest.fixture(scope="module")
+def family(tmp_path_factory):
+    w = plain_random_weights(FAMILY, 4)
+    # larger q/k projections: attention that is not flat (N(0, 0.02) rows of 4096 give scores near 0)
+    w = {k: (v * 4 if ("q_proj" in k or "k_proj" in k) else v).to(torch.bfloat16).float() for k, v in w.items()}
+    folder = save_model_folder(tmp_path_factory.mktemp("family"), FAMILY, w, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(40)
+    tokens = {r: torch.randint(0, FAMILY["vocab_size"], (n,), generator=g).tolist() for r, n in LENGTHS.items()}
+    # sums over 4096 and 14336 terms: the float32 runs are judged against a float64 run
+    exact = {r: plain_forward({k: v.double() for k, v in w.items()}, FAMILY, t, torch.float64).double()
+             for r, t in tokens.items()}
+    plain32 = plain_logits(w, FAMILY, tokens)
+    noise16 = plain_logits(w, FAMILY, tokens, torch.bfloat16)
+    return dict(folder=folder, tokens=tokens, exact=exact, plain32=plain32, noise16=noise16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_family_shape_under_every_cut(family, dtype):
+    for name, trace in (("whole", traces.whole(LENGTHS)), ("tail", traces.tail(LENGTHS, 32)),
+                        ("chunks", traces.chunks(LENGTHS)), ("mixed", traces.mixed(LENGTHS, seed=7, budget=96))):
+        need = traces.max_live_tokens(trace, 64)
+        runner = make_runner(family["folder"], dtype, 64, need)
+        got = run_trace(runner, trace, family["tokens"])
+        if dtype == torch.float32:
+            assert_close(got, family["exact"], dtype, family["plain32"], name)
+        else:
+            assert_close(got, family["plain32"], dtype, family["noise16"], name)
