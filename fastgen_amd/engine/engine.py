@@ -22,7 +22,8 @@ from .scheduler import PlannedEntry, Request, Scheduler
 
 class Engine:
     def __init__(self, model: Model, page_size: int = 64, max_tokens: int = 8192, max_batch: int = 64,
-                 max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0) -> None:
+                 max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0,
+                 sync_freq: int = 10) -> None:
         self.model = model
         self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch)
         cap = getattr(model.args, "max_position", 0) or None
@@ -33,6 +34,9 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit)
         self.sampler = Sampler(model.device)
         self.seed = seed
+        # decode steps between host checks for finished requests when nothing waits for admission
+        # (the reference's GenArgs.sync_freq, fastgen/generate.py:55-59)
+        self.sync_freq = sync_freq
         self._n_requests = 0
         self.n_steps = 0
 
@@ -71,6 +75,9 @@ class Engine:
     def step(self) -> List[Request]:
         """One step of the model over what the scheduler picks; the requests
         that ended with it."""
+        n_run = self.scheduler.plan_decode_run(self.sync_freq) if self.runner.use_graphs else 0
+        if n_run:
+            return self._decode_run(n_run)
         plan = self.scheduler.plan()
         done: List[Request] = []
         if plan:
@@ -99,6 +106,27 @@ class Engine:
                 done.append(r)
         self.scheduler.finished.clear()
         return done
+
+    def _decode_run(self, n_steps: int) -> List[Request]:
+        """``n_steps`` decode steps of all running requests with one look at the
+        tokens at the end."""
+        reqs = list(self.scheduler.running)
+        entries = [StepEntry(r.rid, [r.generated[-1] if r.generated else r.prompt[-1]], [0]) for r in reqs]
+        sample = self.sampler.prepare([r.temperature for r in reqs], [r.top_p for r in reqs],
+                                      [r.seed for r in reqs], [len(r.generated) for r in reqs], n_steps)
+        want_lp = any(r.want_logprobs for r in reqs)
+        lps: List[torch.Tensor] = []
+
+        def sample_and_note(logits, step, out):
+            tok = sample(logits, step, out)
+            if want_lp:
+                lps.append(self.sampler.logprobs(logits, tok))
+            return tok
+
+        out = self.runner.decode_run(entries, n_steps, sample_and_note)
+        tokens = out.tolist()  # the one synchronisation of the run
+        self.n_steps += len(tokens)
+        return self.scheduler.commit_run(tokens, [lp.tolist() for lp in lps] if want_lp else None)
 
     def generate(self, prompts: Sequence[Sequence[int]], params: SamplingParams | Sequence[SamplingParams] = SamplingParams(),
                  ) -> List[List[int]]:
@@ -142,16 +170,21 @@ class Engine:
             self.add_request(p, params)
         while any(r.remaining() > 1 for r in self.scheduler.running) or self.scheduler.waiting:
             self.step()
-        for _ in range(warmup):
-            self.step()
+        def run(n: int) -> None:  # exactly n decode steps, in runs of sync_freq where the engine takes them
+            target = self.n_steps + n
+            keep = self.sync_freq
+            while self.n_steps < target:
+                self.sync_freq = min(keep, target - self.n_steps)
+                if self.step():
+                    raise RuntimeError("time_decode: a request ended inside the measurement")
+            self.sync_freq = keep
+
+        run(warmup)
         if len(self.scheduler.running) != len(prompts) or self.scheduler.n_preemptions:
             raise RuntimeError("time_decode: the batch did not stay whole; give the cache more pages")
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            done = self.step()
-            if done:
-                raise RuntimeError("time_decode: a request ended inside the timed steps")
+        run(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         for r in list(self.scheduler.running):  # the measurement is over: let go of the batch

@@ -37,10 +37,12 @@ class _DecodeGraph:
         model, cache = runner.model, runner.cache
         packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, runner.table_width)
         self.layout = (tuple(int(o) for o in offs), tuple(shapes))
-        self.staging = torch.empty(packed.size, dtype=torch.int32, pin_memory=True)
-        self.staging.numpy()[:] = packed
-        self.packed = self.staging.to(model.device)
-        self.copied = torch.cuda.Event()
+        # a ring of pinned staging buffers: the host may run several steps ahead of the device
+        self.staging = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(runner.run_ahead)]
+        self.copied = [torch.cuda.Event() for _ in range(runner.run_ahead)]
+        self.turn = 0
+        self.staging[0].numpy()[:] = packed
+        self.packed = self.staging[0].to(model.device)
         self.ctx = context_from_packed(self.packed, offs, shapes, host, cache.page_size, model.dtype)
         self.ctx.graph_capacity = runner.table_width * cache.page_size
         # warm up outside the capture (libraries load, the matrix library picks its kernels), then capture
@@ -58,15 +60,22 @@ class _DecodeGraph:
             self.logits = model.forward(self.ctx, runner.stores)
         runner.graph_pool = runner.graph_pool or self.graph.pool()
 
-    def replay(self, runner: "ModelRunner", entries: Sequence[StepEntry]) -> torch.Tensor:
-        packed, offs, shapes, host = pack_context(entries, runner.cache, runner.model.vocab_size,
-                                                  runner.table_width)
+    def replay(self, runner: "ModelRunner", entries: Sequence[StepEntry],
+               tokens_on_device: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Copy the step's vectors in and run the captured step.  With
+        ``tokens_on_device`` (int32 ``[B]``) the tokens come from there, not from
+        ``entries``: the step before sampled them and the host has not seen them."""
+        packed, offs, shapes, host = pack_context(entries, runner.cache, None if tokens_on_device is not None
+                                                  else runner.model.vocab_size, runner.table_width)
         if (tuple(int(o) for o in offs), tuple(shapes)) != self.layout:
             raise RuntimeError("decode graph: the step's layout differs from the captured one")
-        self.copied.synchronize()  # the staging buffer is free again
-        self.staging.numpy()[:] = packed
-        self.packed.copy_(self.staging, non_blocking=True)
-        self.copied.record()
+        i = self.turn = (self.turn + 1) % len(self.staging)
+        self.copied[i].synchronize()  # this staging buffer is free again
+        self.staging[i].numpy()[:] = packed
+        self.packed.copy_(self.staging[i], non_blocking=True)
+        self.copied[i].record()
+        if tokens_on_device is not None:
+            self.ctx.tokens.copy_(tokens_on_device)
         self.graph.replay()
         return self.logits
 
@@ -101,6 +110,7 @@ class ModelRunner:
         self.graphs: Dict[int, _DecodeGraph] = {}
         self.graph_pool = None
         self.max_graphs = 32
+        self.run_ahead = 16  # steps the host may prepare before the device has run them
 
     # ------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> int:
@@ -147,6 +157,30 @@ class ModelRunner:
         return bool(entries) and all(
             len(e.tokens) == 1 and list(e.want) == [0] and self.cache.is_live(e.rid) for e in entries
         ) and (len(entries) in self.graphs or len(self.graphs) < self.max_graphs)
+
+    def decode_run(self, entries: Sequence[StepEntry], n_steps: int, sample) -> torch.Tensor:
+        """``n_steps`` decode steps of the same requests without the host seeing
+        a token in between (``fastgen/generate.py:690-736``: ``sync_freq`` steps
+        between host checks): each step's sampled tokens feed the next on the
+        device.  ``entries`` bring each request's pending token; pages for all
+        steps must be reservable.  ``sample(logits, step, out)`` writes the
+        step's int32 tokens into ``out``.  Returns int32 ``[n_steps, B]`` on
+        the device; the caller reads it once."""
+        if not (self.use_graphs and self._is_plain_decode(entries)):
+            raise RuntimeError("decode_run needs a plain decode step and decode graphs")
+        n_steps = min(n_steps, self.run_ahead - 1)
+        for e in entries:
+            self.cache.reserve(e.rid, n_steps)
+        g = self.graphs.get(len(entries))
+        if g is None:
+            g = self.graphs[len(entries)] = _DecodeGraph(self, entries)
+        out = torch.empty((n_steps, len(entries)), dtype=torch.int32, device=self.model.device)
+        for s in range(n_steps):
+            logits = g.replay(self, entries, out[s - 1] if s else None)
+            sample(logits, s, out[s])
+            for e in entries:
+                self.cache.advance(e.rid, 1)
+        return out
 
     def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         if len({e.rid for e in entries}) != len(entries):

@@ -198,6 +198,57 @@ class Scheduler:
             return self.plan()
         return entries
 
+    # -------------------------------------------------------- decode runs
+    def plan_decode_run(self, max_steps: int) -> int:
+        """How many decode steps all running requests can take in a row without
+        the host looking at a token in between (0: take single steps).  That is
+        when every running request is decoding, nobody waits for a place that a
+        finishing request would free, and no request reaches its length cap or
+        runs out of pages before the run ends.  (The reference runs ``sync_freq``
+        steps when its batch is full, ``fastgen/generate.py:690-699``.)"""
+        if max_steps < 2 or not self.running or self.waiting:
+            return 0
+        n = max_steps
+        for req in self.running:
+            if req.remaining() != 1:
+                return 0
+            n = min(n, req.max_new - len(req.generated), self.max_seq - req.n_known())
+        if n < 2:
+            return 0
+        for g in range(self.cache.n_groups):
+            need = sum(self.cache.pages_needed(r.rid, n)[g] for r in self.running)
+            if need > self.cache.free_pages(g):
+                return 0
+        return n
+
+    def commit_run(self, tokens: Sequence[Sequence[int]], logprobs: Optional[Sequence[Sequence[float]]] = None,
+                   ) -> List[Request]:
+        """Record a decode run: ``tokens[s][b]`` is what running request ``b``
+        sampled at step ``s``.  A request that sampled a stop id ends there; what
+        it sampled afterwards is dropped (``fastgen/generate.py:647-662``)."""
+        done: List[Request] = []
+        n = len(tokens)
+        for b, req in enumerate(list(self.running)):
+            req.n_fed += n
+            reason = None
+            for s in range(n):
+                tok = int(tokens[s][b])
+                req.generated.append(tok)
+                if logprobs is not None and req.want_logprobs:
+                    req.logprobs.append(float(logprobs[s][b]))
+                if tok in req.stop_ids:
+                    reason = "stop"
+                elif len(req.generated) >= req.max_new:
+                    reason = "length"
+                elif req.n_known() >= self.max_seq:
+                    reason = "max_seq"
+                if reason:
+                    break
+            if reason:
+                self._finish(req, reason)
+                done.append(req)
+        return done
+
     # ------------------------------------------------------------- commit
     def commit(self, entries: Sequence[PlannedEntry], sampled: Sequence[int],
                logprobs: Optional[Sequence[float]] = None) -> List[Request]:

@@ -42,6 +42,7 @@ class GenArgs:
     max_prefill: int = 8192  # token budget of one step
     prefill_gb: float = 0.5  # activation budget, used when sizing the cache
     gpu_gb: float = 20  # memory budget, used when max_seq is negative
+    sync_freq: int = 10  # decode steps between host checks for finished requests (when nobody waits)
     seed: int = 777  # the reference's tools seed the global generator with 777 (tools/chat.py:47)
     dtype: torch.dtype = torch.bfloat16
 
@@ -94,7 +95,8 @@ class Fastgen:
         max_batch = max(1, min(gen_args.max_batch, max_seq // gen_args.cache_block))  # generate.py:234-236
         logger.info("cache of %d tokens in pages of %d, at most %d requests", max_seq, gen_args.cache_block, max_batch)
         engine = Engine(model, page_size=gen_args.cache_block, max_tokens=max_seq, max_batch=max_batch,
-                        max_step_tokens=gen_args.max_prefill, max_seq=max_seq, seed=gen_args.seed)
+                        max_step_tokens=gen_args.max_prefill, max_seq=max_seq, seed=gen_args.seed,
+                        sync_freq=gen_args.sync_freq)
         return cls(engine, gen_args, stop_tokens)
 
     def _params(self, pkt: Packet) -> SamplingParams:

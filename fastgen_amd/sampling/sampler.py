@@ -39,14 +39,22 @@ class Sampler:
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
                seeds: Sequence[int], counters: Sequence[int]) -> torch.Tensor:
         """int32 ``[n]`` on the device; row ``i`` is greedy if ``temperatures[i] == 0``."""
-        n = logits.shape[0]
+        return self.prepare(temperatures, top_ps, seeds, counters, 1)(logits, 0, None)
+
+    def prepare(self, temperatures: Sequence[float], top_ps: Sequence[float], seeds: Sequence[int],
+                counters: Sequence[int], n_steps: int):
+        """A function ``(logits, step, out) -> tokens`` for ``n_steps`` steps of
+        the same rows, the parameters copied to the device once; the row's
+        counter at step ``s`` is ``counters[row] + s``."""
         if not any(t > 0 for t in temperatures):
-            return ops.sample(logits)
+            return lambda logits, step, out: ops.sample(logits, out=out)
         packed_f = torch.tensor([list(temperatures), list(top_ps)], dtype=torch.float32).to(self.device)
         mask = (1 << 63) - 1
-        packed_i = torch.tensor([[s & mask for s in seeds], list(counters)], dtype=torch.int64).to(self.device)
+        ints = [[s & mask for s in seeds]] + [[c + s for c in counters] for s in range(n_steps)]
+        packed_i = torch.tensor(ints, dtype=torch.int64).to(self.device)
         top_p = packed_f[1] if any(p < 1.0 for p in top_ps) else None
-        return ops.sample(logits, packed_f[0], top_p, packed_i[0], packed_i[1])
+        return lambda logits, step, out: ops.sample(logits, packed_f[0], top_p, packed_i[0], packed_i[1 + step],
+                                                    out=out)
 
     def logprobs(self, logits: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
         return ops.logprob(logits, tokens)

@@ -265,3 +265,55 @@ def test_random_load_finishes_with_the_right_tokens(seed):
     drive(s)
     for r in reqs:
         assert r.finish_reason == "length" and r.generated == [fake_token(r, len(r.prompt) + i) for i in range(r.max_new)]
+
+
+def test_decode_runs_between_host_checks():
+    """Several decode steps in a row without the host seeing a token (the
+    reference's sync_freq): only when every request decodes, nobody waits,
+    and caps and pages allow it; a stop id inside the run ends the request
+    there and drops what it sampled afterwards."""
+    s = mk(cache_pages=64, max_batch=4, budget=64)
+    a, b = Request("a", [1] * 10, max_new=25), Request("b", [2] * 3, max_new=7)
+    s.add(a), s.add(b)
+    assert s.plan_decode_run(10) == 0  # prompts not fed yet
+    plan = s.plan()
+    for e in plan:
+        s.cache.advance(e.request.rid, e.n)
+    s.commit(plan, [50, 60])
+    assert s.plan_decode_run(10) == 6  # b may take 6 more tokens
+    assert s.plan_decode_run(1) == 0
+    s.add(Request("c", [3], max_new=2))
+    assert s.plan_decode_run(10) == 0  # somebody waits for admission
+    s.waiting.clear()
+    n = s.plan_decode_run(4)
+    assert n == 4
+    for r in (a, b):
+        s.cache.reserve(r.rid, n)
+        s.cache.advance(r.rid, n)
+    a.stop_ids = (77,)
+    done = s.commit_run([[70, 80], [77, 81], [72, 82], [73, 83]])
+    assert done == [a] and a.finish_reason == "stop" and a.generated == [50, 70, 77]
+    assert b.generated == [60, 80, 81, 82, 83] and b.n_fed == 3 + 4 and b.remaining() == 1
+    assert s.plan_decode_run(10) == 2  # b: 7 - 5
+    s.cache.reserve("b", 2), s.cache.advance("b", 2)
+    assert s.commit_run([[90], [91]]) == [b] and b.finish_reason == "length" and len(b.generated) == 7
+    assert s.cache.free_pages() == 64
+    # pages: a run must fit for all requests at once
+    for pages, want in ((4, 10), (3, 0)):
+        t = mk(cache_pages=pages, max_batch=2, budget=64)
+        rs = [Request(i, [1] * 15, max_new=40) for i in range(2)]
+        for r in rs:
+            t.add(r)
+        plan = t.plan()
+        for e in plan:
+            t.cache.advance(e.request.rid, e.n)
+        t.commit(plan, [5, 6])  # both hold 15 tokens in one page; the 17th token needs a second page each
+        assert t.plan_decode_run(10) == want
+    # the cap of one request's length (here the pool itself) bounds a run
+    t = mk(cache_pages=2, max_batch=1, budget=64)
+    r = Request("r", [1] * 28, max_new=50)
+    t.add(r)
+    plan = t.plan()
+    t.cache.advance("r", 28)
+    t.commit(plan, [5])
+    assert t.plan_decode_run(10) == 3

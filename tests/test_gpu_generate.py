@@ -103,6 +103,41 @@ def test_sampled_tokens_follow_the_models_distribution(tiny_b):
     assert chi2 < 2.0 * int(big.sum()) + 30, (float(chi2), int(big.sum()))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_runs_give_the_same_tokens_as_single_steps(tiny_b, dtype):
+    """sync_freq decode steps between host checks (tokens fed back on the
+    device) against one check a step: greedy, seeded sampling, a stop id that
+    falls inside a run, and log-probabilities."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    mk = lambda sf: Engine.from_folder(tiny_b["folder"], dtype, page_size=32, max_tokens=1024, max_batch=4,
+                                       max_step_tokens=256, sync_freq=sf)
+    prompts = tiny_b["prompts"][:4]
+    greedy = SamplingParams(temperature=0.0, max_new_tokens=37)
+    one, many = mk(1), mk(10)
+    want = one.generate(prompts, greedy)
+    got = many.generate(prompts, greedy)
+    assert got == want
+    assert many.n_steps == one.n_steps  # as many model steps, fewer host checks
+    if dtype == torch.float32:
+        assert want == [plain_greedy(tiny_b["weights"], TINY_B, p, 37) for p in prompts]
+    sps = [SamplingParams(temperature=0.9, top_p=0.9, seed=11 + i, max_new_tokens=30, logprobs=True) for i in range(4)]
+    assert mk(10).generate(prompts, sps) == mk(1).generate(prompts, sps)
+    # a stop id in the middle of a run: the request ends with it
+    alone = mk(1).generate([prompts[1]], greedy)[0]
+    stop = alone[20]
+    sp = SamplingParams(temperature=0.0, max_new_tokens=37, stop_ids=(stop,))
+    eng = mk(10)
+    rid = eng.add_request(prompts[1], sp)
+    done = []
+    while eng.has_work():
+        done += eng.step()
+    assert done[0].generated == alone[: alone.index(stop) + 1] and done[0].finish_reason == "stop"
+    assert eng.runner.cache.live_requests() == []
+    eng.runner.cache.check()
+
+
 def test_stop_ids_and_logprobs(tiny_b):
     from fastgen_amd.engine import Engine
     from fastgen_amd.sampling import SamplingParams
