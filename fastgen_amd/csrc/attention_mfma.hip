@@ -103,7 +103,7 @@ struct ItemRows {
 template <bool PREFETCH, int RB, class LK, class LV>
 __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], const bf16x8 (&qop)[RB][NKS],
                                             float scale, float (&m)[RB], float (&l)[RB], f32x4 (&o)[RB][NDB],
-                                            LK load_k, LV load_v) {
+                                            LK load_k, LV load_v, bool all_visible = false) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
   // The order of the loads in the source is the order in which they are issued: all of K, then the
   // first half of V, are in flight before the first MFMA waits for anything; the second half of V is
@@ -144,7 +144,9 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = k0 + key_of(kb, 4 * g + i);
-        const float v = (key >= me[rb].first && key <= me[rb].pos) ? s[rb][kb][i] * scale : -INFINITY;
+        // all_visible (uniform over the wave): every row of the wave sees every key of the tile
+        const float v = (all_visible || (key >= me[rb].first && key <= me[rb].pos)) ? s[rb][kb][i] * scale
+                                                                                   : -INFINITY;
         s[rb][kb][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -408,13 +410,16 @@ constexpr int TILE_RB = HD <= 128 ? 2 : 1;  // row blocks a wave holds (register
 constexpr int TILE_ROWS = 64 * TILE_RB;     // query rows of an item
 
 template <bool PERM>
-__global__ __launch_bounds__(256, 2) void attn_tile_kernel(
+__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
     int page_size, int page_shift, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) bf16_t k_s[TILE * HD];
-  __shared__ __attribute__((aligned(16))) bf16_t v_s[TILE * HD];
+  // two tiles in LDS when they fit in 64 KB: tile i is read while tile i+1 is written and the loads
+  // of tile i+2 are in flight
+  constexpr int NBUF = HD <= 128 ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[NBUF][TILE * HD];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[NBUF][TILE * HD];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int item = blockIdx.x, kvh = blockIdx.y;
@@ -429,6 +434,7 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
   ItemRows me[RB];
   bf16x8 qop[RB][NKS];
   int w_hi = -1, w_lo = 0x7fffffff;  // the keys this wave's rows can see: tiles outside are skipped by the wave
+  int w_all_hi = 0x7fffffff, w_all_lo = 0;  // keys in [w_all_lo, w_all_hi] are seen by all rows of the wave
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = (wave * RB + rb) * 16 + r16;
@@ -440,6 +446,10 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
       me[rb].first = window > 0 && me[rb].pos - window + 1 > 0 ? me[rb].pos - window + 1 : 0;
       w_hi = max(w_hi, me[rb].pos);
       w_lo = min(w_lo, me[rb].first);
+      w_all_hi = min(w_all_hi, me[rb].pos);
+      w_all_lo = max(w_all_lo, me[rb].first);
+    } else {
+      w_all_hi = -1;  // a padding row sees nothing: no tile is all visible
     }
     load_q(qop[rb], q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
   }
@@ -447,6 +457,8 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
   for (int msk = 1; msk < 16; msk <<= 1) {
     w_hi = max(w_hi, __shfl_xor(w_hi, msk, FG_WAVE));
     w_lo = min(w_lo, __shfl_xor(w_lo, msk, FG_WAVE));
+    w_all_hi = min(w_all_hi, __shfl_xor(w_all_hi, msk, FG_WAVE));
+    w_all_lo = max(w_all_lo, __shfl_xor(w_all_lo, msk, FG_WAVE));
   }
 
   float m[RB], l[RB];
@@ -469,6 +481,26 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
   // LDS.  Loads are never conditional: addresses are clamped into the item's key range, value
   // slots outside it are masked, keys outside it give scores that the select discards.
   auto fetch = [&](int k0) {
+    if (PERM && (page_size & 63) == 0 && k0 >= first_min && k0 + TILE - 1 <= pos_last) {
+      // The whole tile lies in one page and inside the key range: K's four 16-key blocks are 64*HD
+      // contiguous elements in the order LDS wants them, V's eight key chunks are a contiguous run
+      // per block of 16 head dims.  No masks, one page lookup.
+      const int kin = pager.in_page(k0);
+      const bf16_t* base_k = k_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)kin * HD;
+      const bf16_t* base_v = v_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)(kin >> 3) * 128;
+      const size_t v_block = (size_t)(page_size >> 3) * 128;  // elements of one block of 16 head dims
+#pragma unroll
+      for (int j = 0; j < KN; ++j) {
+        const int w = min((int)threadIdx.x + 256 * j, KTOT - 1);
+        kreg[j] = *(const bf16x8*)(base_k + (size_t)w * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const int w = min((int)threadIdx.x + 256 * j, VTOT - 1);
+        vreg[j] = *(const bf16x8*)(base_v + (size_t)(w >> 7) * v_block + (size_t)(w & 127) * 8);
+      }
+      return;
+    }
     // K: chunk (block kb, dims 8c.., key r) -> k_s[((kb*KCH + c)*16 + r)*8]; r fastest over threads
 #pragma unroll
     for (int j = 0; j < KN; ++j) {
@@ -510,18 +542,18 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     }
   };
   const int k_first = (first_min / TILE) * TILE;
-  fetch(k_first);
-  for (int k0 = k_first; k0 <= pos_last; k0 += TILE) {
-    __syncthreads();  // the previous tile is no longer read
+  auto stash = [&](int b) {
 #pragma unroll
     for (int j = 0; j < KN; ++j)
-      if (threadIdx.x + 256 * j < KTOT) *(bf16x8*)(k_s + (size_t)(threadIdx.x + 256 * j) * 8) = kreg[j];
+      if (threadIdx.x + 256 * j < KTOT) *(bf16x8*)(k_lds[b] + (size_t)(threadIdx.x + 256 * j) * 8) = kreg[j];
 #pragma unroll
     for (int j = 0; j < VN; ++j)
-      if (threadIdx.x + 256 * j < VTOT) *(bf16x8*)(v_s + (size_t)(threadIdx.x + 256 * j) * 8) = vreg[j];
-    __syncthreads();
-    if (k0 + TILE <= pos_last) fetch(k0 + TILE);  // flies during this tile's MFMAs
-    if (k0 > w_hi || k0 + TILE <= w_lo) continue;  // nothing in this tile for this wave's rows
+      if (threadIdx.x + 256 * j < VTOT) *(bf16x8*)(v_lds[b] + (size_t)(threadIdx.x + 256 * j) * 8) = vreg[j];
+  };
+  auto compute = [&](int k0, int b) {
+    if (k0 > w_hi || k0 + TILE <= w_lo) return;  // nothing in this tile for this wave's rows
+    const bf16_t* k_s = k_lds[b];
+    const bf16_t* v_s = v_lds[b];
     auto load_k = [&](int kb, int ks) -> bf16x8 {
       const int c = 4 * ks + g;
       return c < KCH ? *(const bf16x8*)(k_s + ((kb * KCH + c) * 16 + r16) * 8) : zero8();
@@ -529,7 +561,29 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     auto load_v = [&](int db, int ks) -> bf16x8 {
       return *(const bf16x8*)(v_s + ((db * 8 + 4 * ks + g) * 16 + r16) * 8);
     };
-    attend_tile<false, RB>(k0, me, qop, scale, m, l, o, load_k, load_v);
+    attend_tile<false, RB>(k0, me, qop, scale, m, l, o, load_k, load_v,
+                           k0 >= w_all_lo && k0 + TILE - 1 <= w_all_hi);
+  };
+  if (NBUF == 2) {
+    fetch(k_first);
+    stash(0);
+    if (k_first + TILE <= pos_last) fetch(k_first + TILE);
+    int b = 0;
+    for (int k0 = k_first; k0 <= pos_last; k0 += TILE, b ^= 1) {
+      __syncthreads();  // tile k0 is complete in buffer b; nobody reads buffer b^1 any more
+      if (k0 + TILE <= pos_last) stash(b ^ 1);
+      if (k0 + 2 * TILE <= pos_last) fetch(k0 + 2 * TILE);  // flies during this and the next tile's MFMAs
+      compute(k0, b);
+    }
+  } else {
+    fetch(k_first);
+    for (int k0 = k_first; k0 <= pos_last; k0 += TILE) {
+      __syncthreads();  // the previous tile is no longer read
+      stash(0);
+      __syncthreads();
+      if (k0 + TILE <= pos_last) fetch(k0 + TILE);  // flies during this tile's MFMAs
+      compute(k0, 0);
+    }
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
