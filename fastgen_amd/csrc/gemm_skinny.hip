@@ -15,12 +15,24 @@
 //
 // Replaces the library product of fastgen/forward.py:433-513 where M is small.
 #include "common.h"
+#include "kv_layout.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define EPI_STORE 0
 #define EPI_SILU_MUL 1
+#define EPI_ROPE_KV 2  // w = [q; k; v] projections: rotate q and k, q to y, k and v into their cache pages
+
+// What the EPI_ROPE_KV epilogue needs beside the product (rope_kv.hip does the same as a kernel of
+// its own for steps with more rows).
+struct RopeKv {
+  const float* table;  // [M, rotary_dim/2, 2] cos, sin of each row's position; null: no rotation
+  const int* slots;    // [M] page * page_size + offset of each row's token; < 0: keep k, v out of the cache
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  int n_heads, n_kv, hd, rotary_dim, page_size;
+};
 
 __device__ __forceinline__ bf16x8 gs_zero8() {
   bf16x8 z;
@@ -105,7 +117,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 template <int WAVES, int EPI, class TY>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
-    int ldy, int M, int N, int K) {
+    int ldy, int M, int N, int K, RopeKv rk) {
   constexpr int U = 8;
   __shared__ float red[WAVES][256];
   __shared__ __attribute__((aligned(16))) bf16_t xs[WAVES][4 * U * 16 * 8];  // [k chunk][row][8]
@@ -151,7 +163,49 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
   }
   *(f32x4*)(&red[wave][r16 * 16 + 4 * g]) = acc;
   __syncthreads();
-  if (EPI == EPI_STORE) {
+  if (EPI == EPI_ROPE_KV) {
+    // 16 columns = 8 pairs of one head of q, k or v (head sizes are multiples of 16)
+    for (int e = threadIdx.x; e < 128; e += WAVES * 64) {
+      const int m = e >> 3, p = e & 7, n = n0 + 2 * p;
+      if (m >= M || n >= N) continue;
+      float a = 0.f, b = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) {
+        a += red[wv][m * 16 + 2 * p];
+        b += red[wv][m * 16 + 2 * p + 1];
+      }
+      const int q_cols = rk.n_heads * rk.hd, k_cols = rk.n_kv * rk.hd;
+      const int d = n % rk.hd;
+      if (n < q_cols + k_cols && rk.table && d < rk.rotary_dim) {
+        const float cs = rk.table[((size_t)m * (rk.rotary_dim / 2) + d / 2) * 2];
+        const float sn = rk.table[((size_t)m * (rk.rotary_dim / 2) + d / 2) * 2 + 1];
+        const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+        a = ra;
+        b = rb;
+      }
+      typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+      if (n < q_cols) {
+        bf16x2_t v2 = {(__bf16)a, (__bf16)b};
+        *(bf16x2_t*)((bf16_t*)y + (size_t)m * ldy + n) = v2;
+        continue;
+      }
+      const int slot = rk.slots[m];
+      if (slot < 0) continue;
+      const KvLayout lay(rk.page_size, rk.hd);
+      const int page = slot / rk.page_size, off = slot % rk.page_size;
+      const size_t head_elems = (size_t)rk.page_size * rk.hd;
+      if (n < q_cols + k_cols) {
+        const int kvh = (n - q_cols) / rk.hd;
+        bf16x2_t v2 = {(__bf16)a, (__bf16)b};
+        *(bf16x2_t*)(rk.k_pages + ((size_t)page * rk.n_kv + kvh) * head_elems + lay.k_off(off, d)) = v2;
+      } else {
+        const int kvh = (n - q_cols - k_cols) / rk.hd;
+        bf16_t* vh = rk.v_pages + ((size_t)page * rk.n_kv + kvh) * head_elems;
+        vh[lay.v_off(off, d)] = (bf16_t)a;
+        vh[lay.v_off(off, d + 1)] = (bf16_t)b;
+      }
+    }
+  } else if (EPI == EPI_STORE) {
     for (int e = threadIdx.x; e < 256; e += WAVES * 64) {
       float s = 0.f;
 #pragma unroll
@@ -263,10 +317,10 @@ static void launch_skinny(const void* x, int ldx, const void* w, int ldw, void* 
   if (MB == 1 && M > 1) {  // one row of x is a broadcast already
     if (blocks >= 1024)
       gemm_skinny16_kernel<4, EPI, TY><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K);
+                                                                   (TY*)y, ldy, M, N, K, RopeKv{});
     else
       gemm_skinny16_kernel<8, EPI, TY><<<blocks, 512, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K);
+                                                                   (TY*)y, ldy, M, N, K, RopeKv{});
     return;
   }
   // few blocks: more waves a block, so that enough loads are in flight on every CU
@@ -339,5 +393,30 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   else PICK(4);
 #undef PICK
 #undef GO64
+  return fg_launch_status();
+}
+
+// q, k, v projections of at most 16 rows with the rotation and the cache write in the epilogue:
+// w = [q rows; k rows; v rows] ([(H + 2 KV) * hd, K]); y = rotated q [M, H * hd]; rotated k and v go
+// to slots[m] of the pages.  table: cos/sin of the rows' positions (null: no rotation).
+extern "C" int fg_gemm_skinny_qkv(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int K,
+                                  const float* table, const int* slots, void* k_pages, void* v_pages,
+                                  int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
+                                  hipStream_t stream) {
+  if (M <= 0) return FG_OK;
+  const int N = (n_heads + 2 * n_kv) * hd;
+  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || hd % 16 || n_heads <= 0 ||
+      n_kv <= 0 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 || page_size <= 0 || page_size % 8 ||
+      ldy < n_heads * hd || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table))
+    return FG_ERR_ARG;
+  const RopeKv rk{rotary_dim ? table : nullptr, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
+                  n_heads, n_kv, hd, rotary_dim, page_size};
+  const int blocks = N / 16;
+  if (blocks >= 1024)
+    gemm_skinny16_kernel<4, EPI_ROPE_KV, bf16_t><<<blocks, 256, 0, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk);
+  else
+    gemm_skinny16_kernel<8, EPI_ROPE_KV, bf16_t><<<blocks, 512, 0, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk);
   return fg_launch_status();
 }

@@ -437,6 +437,37 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     return y
 
 
+def gemm_skinny_qkv(x: torch.Tensor, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots: torch.Tensor,
+                    k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                    rotary_dim: int) -> torch.Tensor:
+    """The q, k, v projections of at most 16 rows with :func:`rope_kv_write` in
+    the product's epilogue: returns the rotated queries ``[M, H*hd]``; the rotated
+    keys and the values go straight into their cache pages."""
+    _gpu(x, wqkv, table, slots, k_pages, v_pages)
+    M, K = x.shape
+    _need(x.dtype == torch.bfloat16 and wqkv.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
+          and v_pages.dtype == torch.bfloat16, "gemm_skinny_qkv takes bfloat16")
+    _need(0 < M <= 16 and wqkv.shape == ((n_heads + 2 * n_kv) * head_dim, K), "x [M<=16, K], wqkv [(H+2KV)*hd, K]")
+    _need(K % 8 == 0 and x.stride(1) == 1 and wqkv.stride(1) == 1 and x.stride(0) % 8 == 0
+          and wqkv.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and wqkv.data_ptr() % 16 == 0,
+          "K must be a multiple of 8, rows 16-byte aligned")
+    _need(head_dim % 16 == 0, "head size must be a multiple of 16")
+    page_size = k_pages.shape[2]
+    _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.shape[1:] == (n_kv, page_size, head_dim)
+          and v_pages.shape == (k_pages.shape[0], n_kv, head_dim, page_size), "pages do not fit the heads")
+    _i32(slots, "slots", M)
+    if rotary_dim:
+        _need(table is not None and table.dtype == torch.float32 and table.is_contiguous()
+              and table.shape == (M, rotary_dim // 2, 2), "table must be float32 [M, rotary_dim/2, 2]")
+    q = torch.empty((M, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    st = _lib.load("gemm_skinny").fg_gemm_skinny_qkv(
+        _ptr(x), x.stride(0), _ptr(wqkv), wqkv.stride(0), _ptr(q), q.stride(0), M, K,
+        _ptr(table if rotary_dim else None), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_heads, n_kv, head_dim,
+        rotary_dim, page_size, _stream(x))
+    _check(st, "gemm_skinny_qkv")
+    return q
+
+
 # ------------------------------------------------------------------- sampling
 def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
            top_p: Optional[torch.Tensor] = None, seeds: Optional[torch.Tensor] = None,

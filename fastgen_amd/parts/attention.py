@@ -13,7 +13,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear
+from ..kernels.linear import linear, skinny_ok
 from .base import LayerStore, Mixer, PagedNeed, TensorSpec, build_part, place, register_part, MATRIX
 
 
@@ -62,9 +62,6 @@ class Attention(Mixer):
     def forward(self, x: torch.Tensor, ctx: Any, store: LayerStore) -> torch.Tensor:
         group = ctx.groups[store.group]
         q_width = self.n_heads * self.head_dim
-        # an entry that reads another entry's cache needs its queries only
-        w = self.wqkv if store.owns else self.wqkv[:q_width]
-        qkv = linear(x, w)
         table = None
         if self.freqs is not None:
             # sin and cos of the step's positions: computed by the first layer, shared by all layers
@@ -73,11 +70,18 @@ class Attention(Mixer):
             table = ctx.scratch.get(key)
             if table is None:
                 table = ctx.scratch[key] = ops.rope_table(ctx.positions, self.freqs)
-        ops.rope_kv_write(
-            qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
-            self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
-            table=table,
-        )
+        if store.owns and self.head_dim % 16 == 0 and skinny_ok(x, self.wqkv):
+            # few rows (decode): rotation and cache write happen where the product is stored
+            qkv = ops.gemm_skinny_qkv(x, self.wqkv, table, group.slots, store.k_pages, store.v_pages, self.n_heads,
+                                      self.n_kv_heads, self.head_dim, self.position.rotary_dim)
+        else:
+            # an entry that reads another entry's cache needs its queries only
+            qkv = linear(x, self.wqkv if store.owns else self.wqkv[:q_width])
+            ops.rope_kv_write(
+                qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
+                self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
+                table=table,
+            )
         out = torch.empty((x.shape[0], q_width), dtype=x.dtype, device=x.device)
         ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,
                             self.window or 0)

@@ -149,6 +149,49 @@ def test_rope_kv_write(ops, dtype, H, KV, hd, rot, P, with_table):
     assert torch.equal(unpack_v(vp_d.cpu()), want_v)  # nothing else in the pool changed either
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("H,KV,hd,rot,P,K", [(4, 2, 16, 16, 16, 64), (5, 1, 48, 48, 32, 240), (8, 2, 128, 128, 64, 1024),
+                                             (6, 3, 64, 32, 8, 328), (3, 3, 80, 0, 16, 72)])
+def test_gemm_skinny_qkv_rotates_and_writes_the_cache(ops, M, H, KV, hd, rot, P, K):
+    """The decode step's fused product: the same result as the product, the
+    rotation and the cache write as three steps (plain fp32 arithmetic here)."""
+    torch.manual_seed(M + hd)
+    n_pages = 5
+    x = (torch.randn(M, K) * 0.5).to(torch.bfloat16)
+    w = (torch.randn((H + 2 * KV) * hd, K) * K**-0.5).to(torch.bfloat16)
+    pos = torch.randint(0, 5000, (M,), dtype=torch.int32)
+    freqs = plain_rope_frequencies(rot, 10000.0) if rot else None
+    slots = torch.randperm(n_pages * P)[:M].to(torch.int32)
+    if M > 2:
+        slots[2] = -1
+    kp_d = torch.full((n_pages, KV, P, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    vp_d = torch.full((n_pages, KV, hd, P), 7.0, dtype=torch.bfloat16, device=DEV)
+    table = ops.rope_table(pos.to(DEV), freqs.to(DEV)) if rot else None
+    got_q = ops.gemm_skinny_qkv(x.to(DEV), w.to(DEV), table, slots.to(DEV), kp_d, vp_d, H, KV, hd, rot).cpu()
+    qkv = x.float() @ w.float().T
+    q = qkv[:, : H * hd].view(M, H, hd)
+    k = qkv[:, H * hd : (H + KV) * hd].view(M, KV, hd)
+    v = qkv[:, (H + KV) * hd :].view(M, KV, hd)
+
+    def rotate(t):
+        if not rot:
+            return t
+        out = t.clone()
+        out[..., :rot] = plain_rope_interleaved(t[..., :rot], pos, freqs)
+        return out
+
+    assert torch.allclose(got_q.float(), rotate(q).reshape(M, -1), **tol(torch.bfloat16))
+    want_k, want_v = torch.full((n_pages, KV, P, hd), 7.0), torch.full((n_pages, KV, P, hd), 7.0)
+    rk = rotate(k)
+    for t in range(M):
+        s = int(slots[t])
+        if s >= 0:
+            want_k[s // P, :, s % P, :] = rk[t]
+            want_v[s // P, :, s % P, :] = v[t]
+    assert torch.allclose(unpack_k(kp_d.cpu()).float(), want_k, **tol(torch.bfloat16))
+    assert torch.allclose(unpack_v(vp_d.cpu()).float(), want_v, **tol(torch.bfloat16))
+
+
 # ---------------------------------------------------------------- attention
 def _paged_case(dtype, seqs, H, KV, hd, P, seed, poison=True, peak=None):
     """``seqs``: list of (n_cached, n_new).  Returns device operands and the
