@@ -63,6 +63,8 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+#define LOG2E 1.4426950408889634f
+
 // key (within a tile) of S^T row `row` (0..15) of key block kb (0..3)
 __device__ __forceinline__ int key_of(int kb, int row) { return 16 * kb + row; }
 
@@ -100,10 +102,12 @@ struct ItemRows {
 // before anything is computed (more registers).  Otherwise (operands in LDS)
 // each is read where it is used.  RB: blocks of 16 query rows a wave holds;
 // every K and V operand it reads serves all of them.
-template <bool PREFETCH, int RB, class LK, class LV>
+// ALLVIS: every row of the wave sees every key of the tile (no mask is computed).
+// scale_log2 = scale * log2(e): scores, running maxima and exponents are kept in base 2.
+template <bool PREFETCH, int RB, bool ALLVIS, class LK, class LV>
 __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], const bf16x8 (&qop)[RB][NKS],
-                                            float scale, float (&m)[RB], float (&l)[RB], f32x4 (&o)[RB][NDB],
-                                            LK load_k, LV load_v, bool all_visible = false) {
+                                            float scale_log2, float (&m)[RB], float (&l)[RB], f32x4 (&o)[RB][NDB],
+                                            LK load_k, LV load_v) {
   const int g = (threadIdx.x % FG_WAVE) >> 4;
   // The order of the loads in the source is the order in which they are issued: all of K, then the
   // first half of V, are in flight before the first MFMA waits for anything; the second half of V is
@@ -143,31 +147,36 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = k0 + key_of(kb, 4 * g + i);
-        // all_visible (uniform over the wave): every row of the wave sees every key of the tile
-        const float v = (all_visible || (key >= me[rb].first && key <= me[rb].pos)) ? s[rb][kb][i] * scale
-                                                                                   : -INFINITY;
+        float v = s[rb][kb][i];  // unscaled: the scale is positive, so it commutes with the maximum
+        if (!ALLVIS) {
+          const int key = k0 + key_of(kb, 4 * g + i);
+          // bitwise, not short-circuit: a select, no branch
+          v = ((key >= me[rb].first) & (key <= me[rb].pos)) ? v : -INFINITY;
+        }
         s[rb][kb][i] = v;
         mx = fmaxf(mx, v);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, FG_WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, FG_WAVE));
-    const float m_new = fmaxf(m[rb], mx);
+    const float m_new = fmaxf(m[rb], mx * scale_log2);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-    const float alpha = __expf(m[rb] - m_use);             // m = -inf: 0
+    const float alpha = __builtin_amdgcn_exp2f(m[rb] - m_use);  // m = -inf: 0
     float sum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = __expf(s[rb][kb][i] - m_use);
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[rb][kb][i], scale_log2, -m_use));
         sum += p;
         pop[rb][kb >> 1][4 * (kb & 1) + i] = (__bf16)p;
       }
     l[rb] = l[rb] * alpha + sum;  // this lane's share of the row's sum; the groups are added at the end
-    m[rb] = m_new;
+    // once the maxima have settled no row of the wave changes its maximum: nothing to rescale then
+    if (__builtin_amdgcn_ballot_w64(m_new != m[rb]) != 0) {
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) o[rb][db] *= alpha;
+      for (int db = 0; db < NDB; ++db) o[rb][db] *= alpha;
+    }
+    m[rb] = m_new;
   }
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks)
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
       }
       return and_mask(v, vmask[ks]);
     };
-    attend_tile<true, 1>(k0, me, qop, scale, m_, l_, o_, load_k, load_v);
+    attend_tile<true, 1, false>(k0, me, qop, scale * LOG2E, m_, l_, o_, load_k, load_v);
   }
   float m = m_[0], l = l_[0];
   f32x4(&o)[NDB] = o_[0];
@@ -308,8 +317,8 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   auto take = [&](int slot) {
     const float mo = ml_s[slot][r16][0], lo = ml_s[slot][r16][1];
     const float M = fmaxf(m, mo);
-    const float fs = m == -INFINITY ? 0.f : __expf(m - M);
-    const float fo = mo == -INFINITY ? 0.f : __expf(mo - M);
+    const float fs = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);  // maxima are in base 2
+    const float fo = mo == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mo - M);
     l = fs * l + fo * lo;
     m = M;
 #pragma unroll
@@ -363,7 +372,7 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
   for (int s = 0; s < n_splits; ++s) {
     const size_t row = row0 + (size_t)s * 16;
     const float ms = part_ml[row * 2];
-    const float f = ms == -INFINITY ? 0.f : __expf(ms - M);
+    const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);  // the splits' maxima are in base 2
     L += f * part_ml[row * 2 + 1];
     O += f * part_o[row * HD + d];
   }
@@ -385,7 +394,7 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
                              int hd, int page_size, float scale, int window, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
-      n_splits < 1 || n_splits > 65535 || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
+      !(scale > 0.f) || n_splits < 1 || n_splits > 65535 || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
       out_stride % 4 || (n_splits > 1 && (!part_o || !part_ml)))
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                           \
@@ -402,7 +411,7 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
 }
 
 // ------------------------------------------------------------------- tile
-// grid (n_items, n_kv), 256 threads: 4 waves of TILE_RB x 16 rows; an item has
+// grid n_items * n_kv, 256 threads: 4 waves of TILE_RB x 16 rows; an item has
 // at most TILE_ROWS / (H / KV) tokens.  The K and V tiles go through LDS in the order the
 // operands are read: K [4 key blocks][HD/8 chunks][16 keys][8], V [HD/16 dim
 // blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
@@ -413,8 +422,8 @@ template <bool PERM>
 __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
-    int page_size, int page_shift, float scale, int window) {
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_items, int n_heads,
+    int n_kv, int page_size, int page_shift, float scale, int window) {
   // two tiles in LDS when they fit in 64 KB: tile i is read while tile i+1 is written and the loads
   // of tile i+2 are in flight
   constexpr int NBUF = HD <= 128 ? 2 : 1;
@@ -422,7 +431,12 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[NBUF][TILE * HD];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
-  const int item = blockIdx.x, kvh = blockIdx.y;
+  // (item, kv head) pairs in launch order: the first half ascending, the second half descending.
+  // Workgroups are handed out in order and a compute unit holds two, so where the items are the
+  // pieces of one prompt (work grows with the position) a late piece shares its unit with an early one.
+  const int n_pairs = gridDim.x, half = (n_pairs + 1) / 2;
+  const int pair = (int)blockIdx.x < half ? (int)blockIdx.x : n_pairs - 1 - ((int)blockIdx.x - half);
+  const int item = pair % n_items, kvh = pair / n_items;
   const int G = n_heads / n_kv;
   const Item it = load_item(items, item);
   const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
@@ -561,8 +575,10 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
     auto load_v = [&](int db, int ks) -> bf16x8 {
       return *(const bf16x8*)(v_s + ((db * 8 + 4 * ks + g) * 16 + r16) * 8);
     };
-    attend_tile<false, RB>(k0, me, qop, scale, m, l, o, load_k, load_v,
-                           k0 >= w_all_lo && k0 + TILE - 1 <= w_all_hi);
+    if (k0 >= w_all_lo && k0 + TILE - 1 <= w_all_hi)  // uniform over the wave
+      attend_tile<false, RB, true>(k0, me, qop, scale * LOG2E, m, l, o, load_k, load_v);
+    else
+      attend_tile<false, RB, false>(k0, me, qop, scale * LOG2E, m, l, o, load_k, load_v);
   };
   if (NBUF == 2) {
     fetch(k_first);
@@ -610,13 +626,13 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
                             int n_items, int n_heads, int n_kv, int hd, int page_size, float scale, int window,
                             hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
-  if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > TILE_ROWS || page_size < 8 || page_size % 8 ||
-      n_kv > 65535 || window < 0 || q_stride % 8 || out_stride % 4)
+  if (hd != HD || !(scale > 0.f) || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > TILE_ROWS || page_size < 8 || page_size % 8 ||
+      (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                        \
-  attn_tile_kernel<PERM><<<dim3(n_items, n_kv), 256, 0, stream>>>(                                          \
+  attn_tile_kernel<PERM><<<n_items * n_kv, 256, 0, stream>>>(                                               \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
-      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
+      block_table, bt_stride, items, n_items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
   if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
 #undef LAUNCH
   return fg_launch_status();

@@ -28,6 +28,21 @@ __device__ __forceinline__ float uniform01(uint64_t seed, uint64_t counter) {
   return (float)(z >> 40) * (1.0f / 16777216.0f);
 }
 
+// f(i, x[i]) for this thread's share of a row (i = tid, tid + threads, ... in ascending order), with
+// eight loads in flight at a time: a row is read by one workgroup, so latency is what it costs.
+template <class F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ x, int vocab, F f) {
+  int i = threadIdx.x;
+  for (; i + 7 * SMP_THREADS < vocab; i += 8 * SMP_THREADS) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = x[i + u * SMP_THREADS];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) f(i + u * SMP_THREADS, v[u]);
+  }
+  for (; i < vocab; i += SMP_THREADS) f(i, x[i]);
+}
+
 // (value, index) maximum with the lowest index winning ties; every thread
 // gets the result.
 __device__ __forceinline__ void block_argmax(float& v, int& idx, float* lds_v, int* lds_i) {
@@ -71,13 +86,12 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
 
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = tid; i < vocab; i += SMP_THREADS) {
-    const float v = x[i];
+  for_each_logit(x, vocab, [&](int i, float v) {
     if (v > best) {  // ascending i: the first maximum is kept
       best = v;
       best_i = i;
     }
-  }
+  });
   block_argmax(best, best_i, red_v, red_i);
   const float temp = temperature ? temperature[r] : 0.f;
   if (!(temp > 0.f)) {
@@ -87,7 +101,7 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
   const float inv_t = 1.f / temp;
   const float mx = best;
   float z = 0.f;
-  for (int i = tid; i < vocab; i += SMP_THREADS) z += expf((x[i] - mx) * inv_t);
+  for_each_logit(x, vocab, [&](int, float v) { z += expf((v - mx) * inv_t); });
   z = block_sum(z, red_v);
 
   // ---- nucleus: smallest weight that is kept
@@ -100,10 +114,10 @@ __global__ __launch_bounds__(SMP_THREADS) void sample_kernel(
       const unsigned mid = lo + (hi - lo) / 2u;
       const float xm = __uint_as_float(mid);
       float mass = 0.f;
-      for (int i = tid; i < vocab; i += SMP_THREADS) {
-        const float w = expf((x[i] - mx) * inv_t);
+      for_each_logit(x, vocab, [&](int, float v) {
+        const float w = expf((v - mx) * inv_t);
         if (w > xm) mass += w;
-      }
+      });
       mass = block_sum(mass, red_v);
       if (mass <= budget) hi = mid; else lo = mid;
     }
@@ -191,10 +205,10 @@ __global__ __launch_bounds__(SMP_THREADS) void logprob_kernel(
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* x = logits + (size_t)r * ld;
   float mx = -INFINITY;
-  for (int i = tid; i < vocab; i += SMP_THREADS) mx = fmaxf(mx, x[i]);
+  for_each_logit(x, vocab, [&](int, float v) { mx = fmaxf(mx, v); });
   mx = block_max(mx, red);
   float z = 0.f;
-  for (int i = tid; i < vocab; i += SMP_THREADS) z += expf(x[i] - mx);
+  for_each_logit(x, vocab, [&](int, float v) { z += expf(v - mx); });
   z = block_sum(z, red);
   if (tid == 0) {
     int tok = tokens[r];
