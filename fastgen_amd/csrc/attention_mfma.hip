@@ -357,27 +357,55 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   }
 }
 
-// grid (16 rows, n_kv, n_items), one thread per head dimension
+// grid (16 rows, n_kv, n_items), one thread per head dimension (at least one wave).  The splits'
+// maxima and sums are read by the first wave, one split a lane, and the partial outputs eight at a
+// time: the kernel is a chain of dependent reads, so what it costs is how long that chain is.
+#define COMBINE_MAX_SPLITS 256
 __global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     const int* __restrict__ items, bf16_t* __restrict__ out, int out_stride,
                                     int n_heads, int n_kv, int n_splits) {
+  __shared__ float f_s[COMBINE_MAX_SPLITS];  // weight of each split's partial output: 2^(m_s - M) / L
   const int r = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z, d = threadIdx.x;
   const int G = n_heads / n_kv;
   const Item it = load_item(items, item);
-  if (r >= it.n_tok * G || d >= HD) return;
+  if (r >= it.n_tok * G) return;  // the whole workgroup
   const size_t row0 = (((size_t)item * n_kv + kvh) * n_splits) * 16 + r;
-  float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(row0 + (size_t)s * 16) * 2]);
-  float L = 0.f, O = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const size_t row = row0 + (size_t)s * 16;
-    const float ms = part_ml[row * 2];
-    const float f = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);  // the splits' maxima are in base 2
-    L += f * part_ml[row * 2 + 1];
-    O += f * part_o[row * HD + d];
+  if (threadIdx.x < FG_WAVE) {
+    constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
+    float ms[PER], ls[PER];
+    float M = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int sp = threadIdx.x + j * FG_WAVE;
+      const float2 ml = *(const float2*)(part_ml + (row0 + (size_t)min(sp, n_splits - 1) * 16) * 2);
+      ms[j] = sp < n_splits ? ml.x : -INFINITY;  // maxima are in base 2
+      ls[j] = ml.y;
+      M = fmaxf(M, ms[j]);
+    }
+    M = wave_max(M);
+    float L = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      ms[j] = ms[j] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[j] - M);
+      L += ms[j] * ls[j];
+    }
+    L = wave_sum(L);
+    const float inv = 1.f / L;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) f_s[threadIdx.x + j * FG_WAVE] = ms[j] * inv;
+  }
+  __syncthreads();
+  if (d >= HD) return;
+  float O = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = part_o[(row0 + (size_t)min(s0 + u, n_splits - 1) * 16) * HD + d];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) O += (s0 + u < n_splits ? f_s[s0 + u] : 0.f) * v[u];
   }
   const int t = it.tok0 + r / G, h = kvh * G + r % G;
-  out[(size_t)t * out_stride + (size_t)h * HD + d] = (bf16_t)(O / L);
+  out[(size_t)t * out_stride + (size_t)h * HD + d] = (bf16_t)O;
 }
 
 static int page_shift_of(int page_size) {
@@ -394,7 +422,7 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
                              int hd, int page_size, float scale, int window, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
-      !(scale > 0.f) || n_splits < 1 || n_splits > 65535 || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
+      !(scale > 0.f) || n_splits < 1 || n_splits > COMBINE_MAX_SPLITS || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
       out_stride % 4 || (n_splits > 1 && (!part_o || !part_ml)))
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                           \

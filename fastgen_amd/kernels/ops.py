@@ -9,7 +9,10 @@ is not on a GPU is refused.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
+
+import numpy as np
 
 import torch
 
@@ -244,13 +247,12 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
 
 
 MFMA_MAX_HEAD_DIM = 256
-import os as _os
 
 # Workgroups wanted for the decode attention kernel: one per CU measured best (256 CUs; 128 to 2048
 # tried at batch 1, 8 and 64).  The splits' partial results are merged by a second kernel: merging
 # them in the split that finishes last needs device-scope fences, which on a GPU of several
 # dies cost more than the launch they save (measured).
-_SPLIT_TARGET_BLOCKS = int(_os.environ.get("FG_SPLIT_TARGET", 256))
+_SPLIT_TARGET_BLOCKS = int(os.environ.get("FG_SPLIT_TARGET", 256))
 
 
 def attention_tile_rows(head_dim: int) -> int:
@@ -264,10 +266,9 @@ def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int =
     Returns two int32 arrays ``[n, 4]`` of (sequence, first flat token, tokens,
     position of the first token): items of at most 16 rows for the split
     kernel (decoded tokens and very short portions) and items of at most
-    ``tile_rows`` rows for the tile kernel, those with the most keys first.
+    ``tile_rows`` rows for the tile kernel, those with the most keys first (the
+    kernel starts them in that order and pairs the first with the last).
     """
-    import numpy as np
-
     small, big = [], []
     per_tile = max(1, tile_rows // group_size)
     for b, n in enumerate(q_lens):
@@ -296,6 +297,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     _need(k_pages.is_contiguous() and v_pages.is_contiguous() and v_pages.shape == (n_pages, n_kv, hd, page_size),
           "k_pages [n_pages, KV, P, hd] and v_pages [n_pages, KV, hd, P] must be contiguous")
     _need(n_heads % n_kv == 0 and page_size % 8 == 0, "heads must be a multiple of kv heads, pages of 8 tokens")
+    _need(scale > 0, "the score scale must be positive")
     T = q.shape[0]
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * hd and q.stride(0) % 8 == 0
           and q.data_ptr() % 16 == 0, "q must be [T, >= H*hd], rows 16-byte aligned")
@@ -351,8 +353,6 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
                                        ctx.positions, n_heads, scale, window)
     plan = ctx.scratch.get(("attention_items", G))
     if plan is None:
-        import numpy as np
-
         if ctx.seq_records is not None and int(ctx.q_lens.max()) * G <= 16:
             # every sequence is one item of the split kernel: its records are in the step's buffer
             # already (and are refreshed with it when the step is a replayed graph)
@@ -444,6 +444,7 @@ def gemm_skinny_qkv(x: torch.Tensor, wqkv: torch.Tensor, table: Optional[torch.T
     the product's epilogue: returns the rotated queries ``[M, H*hd]``; the rotated
     keys and the values go straight into their cache pages."""
     _gpu(x, wqkv, table, slots, k_pages, v_pages)
+    _need(x.dim() == 2 and wqkv.dim() == 2 and k_pages.dim() == 4, "x [M, K], wqkv [N, K], k_pages [n, KV, P, hd]")
     M, K = x.shape
     _need(x.dtype == torch.bfloat16 and wqkv.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
           and v_pages.dtype == torch.bfloat16, "gemm_skinny_qkv takes bfloat16")
