@@ -113,7 +113,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 // MFMA operand row group reads 16 different rows of x, which from memory is 16
 // cache lines for 256 bytes; instead the wave copies its 16 x 256 slice of x
 // for the next 8 k steps with whole-row loads into LDS, chunk-major, and reads
-// the operands from there (the 16 lanes then read 256 contiguous bytes).
+// the operands from there (the 16 lanes then read 256 contiguous bytes).  Row r
+// of chunk c sits in slot r ^ (c & 15) of the chunk: the 16 lanes that store one
+// row's consecutive chunks would otherwise all hit the same banks (a chunk is
+// 256 bytes, the width of all banks).
 template <int WAVES, int EPI, class TY>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
@@ -152,12 +155,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     __builtin_amdgcn_wave_barrier();  // the reads of the previous iteration are done (same wave, in order)
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      if (j < x_loads) *(bf16x8*)(my_xs + (c_chunk * 16 + 2 * j + c_row) * 8) = xv[j];
+      if (j < x_loads) *(bf16x8*)(my_xs + (c_chunk * 16 + ((2 * j + c_row) ^ (c_chunk & 15))) * 8) = xv[j];
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const bf16x8 b = *(const bf16x8*)(my_xs + ((4 * u + g) * 16 + r16) * 8);
+      const bf16x8 b = *(const bf16x8*)(my_xs + ((4 * u + g) * 16 + (r16 ^ ((4 * u + g) & 15))) * 8);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc, 0, 0, 0);
     }
   }
@@ -233,12 +236,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
 // goes through LDS once for all four waves.  blockIdx.y cuts K: split s adds
 // rows k in [s*k_per_split, ...) and stores its partial sums at y + s *
 // part_stride (fp32); the consumer adds the partials in split order.
-template <int MB, int EPI, class TY>
-__global__ __launch_bounds__(256) void gemm_skinny64_kernel(
+// U: k steps of 32 a pass of the loop (8; 4 halves the x slice in LDS and doubles the workgroups a CU
+// holds, which measured no faster at 64 rows).
+template <int MB, int U, int EPI, class TY>
+__global__ __launch_bounds__(256, U == 4 ? 4 : 2) void gemm_skinny64_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
     int ldy, size_t part_stride, int M, int N, int K, int k_per_split) {
-  constexpr int U = 8;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][4 * U * MB * 16 * 8];  // [buffer][k chunk][row][8]
+  // [buffer][k chunk][row][8]; row r of chunk c in slot r ^ (c & 15) of its block of 16 (bank conflicts, as above)
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][4 * U * MB * 16 * 8];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 64 + wave * 16;
@@ -247,16 +252,17 @@ __global__ __launch_bounds__(256) void gemm_skinny64_kernel(
   f32x4 acc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // copying x: 32 chunks a row and iteration; thread t copies chunk t % 32 of rows t / 32 + 8 j
-  const int c_chunk = threadIdx.x & 31, c_row = threadIdx.x >> 5;
-  constexpr int XL = MB * 2;  // loads a thread issues for the x slice
+  // copying x: 4 U chunks a row and pass; thread t copies chunk t % (4 U) of rows t / (4 U) + RP j
+  constexpr int RP = 256 / (4 * U);  // rows the workgroup copies at a time
+  const int c_chunk = threadIdx.x & (4 * U - 1), c_row = threadIdx.x / (4 * U);
+  constexpr int XL = MB * 16 / RP;  // loads a thread issues for the x slice
   // The loads of the next 8 k steps (W and the x slice) are in flight while the current ones are
   // multiplied: they are issued right after the barrier that publishes the current x slice.
   bf16x8 a_next[U], xv[XL];
   auto fetch = [&](int kk) {
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
-      const int row = min(c_row + 8 * j, M - 1), k = kk + 8 * c_chunk;
+      const int row = min(c_row + RP * j, M - 1), k = kk + 8 * c_chunk;
       xv[j] = *(const bf16x8*)(x + (size_t)row * ldx + (k < k_end ? k : k_begin));
     }
 #pragma unroll
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(256) void gemm_skinny64_kernel(
   for (int kk = k_begin; kk < k_end; kk += 32 * U, buf ^= 1) {
     bf16_t* my = xs[buf];
 #pragma unroll
-    for (int j = 0; j < XL; ++j) *(bf16x8*)(my + (c_chunk * (MB * 16) + c_row + 8 * j) * 8) = xv[j];
+    for (int j = 0; j < XL; ++j) *(bf16x8*)(my + (c_chunk * (MB * 16) + ((c_row + RP * j) ^ (c_chunk & 15))) * 8) = xv[j];
     bf16x8 a[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) a[u] = a_next[u];
@@ -282,7 +288,7 @@ __global__ __launch_bounds__(256) void gemm_skinny64_kernel(
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const bf16x8 b = *(const bf16x8*)(my + ((4 * u + g) * (MB * 16) + 16 * mb + r16) * 8);
+        const bf16x8 b = *(const bf16x8*)(my + ((4 * u + g) * (MB * 16) + 16 * mb + (r16 ^ ((4 * u + g) & 15))) * 8);
         acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b, acc[mb], 0, 0, 0);
       }
   }
@@ -377,9 +383,9 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   const int k_per_split = ((K + k_splits * 256 - 1) / (k_splits * 256)) * 256;
   const dim3 grid((N + 63) / 64, k_splits);
   const int mb = (M + 15) / 16;
-#define GO64(MB, EPI, TY)                                                                              \
-  gemm_skinny64_kernel<MB, EPI, TY><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, \
-                                                              ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split)
+#define GO64(MB, EPI, TY)                                                                                    \
+  gemm_skinny64_kernel<MB, 8, EPI, TY><<<grid, 256, 0, stream>>>(                             \
+      (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split)
 #define PICK(MB)                                                                   \
   do {                                                                             \
     if (epilogue == EPI_SILU_MUL) GO64(MB, EPI_SILU_MUL, bf16_t);                  \
