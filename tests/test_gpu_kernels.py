@@ -556,11 +556,13 @@ def test_paged_attention_mfma_window_edge(ops):
             assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs, w), atol=1.5e-2, rtol=2e-2)
 
 
-def test_paged_attention_mfma_long_context(ops):
+@pytest.mark.parametrize("n_splits", [16, 64, 200])
+def test_paged_attention_mfma_long_context(ops, n_splits):
     """Llama-3.1-8B's attention shape at a context of several thousand keys,
-    one decoded token and one long portion."""
+    one decoded token and one long portion; with more splits than one wave
+    of the combine has lanes, and more splits than the short sequence has tiles."""
     H, KV, hd, P = 32, 8, 128, 64
-    seqs = [(5000, 1), (3000, 200)]
+    seqs = [(5000, 1), (3000, 200), (70, 1)]
     case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=24, poison=True)
-    out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, 16)
+    out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, n_splits)
     assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
