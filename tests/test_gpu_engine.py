@@ -101,6 +101,31 @@ def test_token_by_token_from_the_first(case, dtype):
     assert_close(got, {rid: case["want"][rid]}, dtype, case["noise"], "one-by-one")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_of_a_batch(dtype, tmp_path):
+    """Three requests decode together for hundreds of steps (the captured decode
+    step is replayed while block tables grow over dozens of small pages and the
+    requests end one after the other), every position against the plain run."""
+    cfg = TINY_C
+    weights = sharpen(plain_random_weights(cfg, 7))
+    weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    folder = save_model_folder(tmp_path / "long", cfg, weights)
+    prompt = {"a": 20, "b": 35, "c": 7}
+    lengths = {"a": 500, "b": 420, "c": 300}
+    g = torch.Generator().manual_seed(11)
+    tokens = {rid: torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for rid, n in lengths.items()}
+    trace = [([(rid, 0, n)], []) for rid, n in prompt.items()]
+    at = dict(prompt)
+    while at:
+        trace.append(([(rid, p, 1) for rid, p in at.items()], [rid for rid, p in at.items() if p + 1 == lengths[rid]]))
+        at = {rid: p + 1 for rid, p in at.items() if p + 1 < lengths[rid]}
+    runner = make_runner(folder, dtype, 16, sum(-(-n // 64) * 64 for n in lengths.values()))
+    got = run_trace(runner, trace, tokens)
+    assert runner.cache.live_requests() == []
+    noise = plain_logits(weights, cfg, tokens, torch.bfloat16) if dtype == torch.bfloat16 else None
+    assert_close(got, plain_logits(weights, cfg, tokens), dtype, noise, "long decoding")
+
+
 def test_float32_does_not_depend_on_the_cut(case):
     """In 32-bit the logits at a position are the same numbers however the
     tokens were cut and batched (every reduction runs in an order fixed by
