@@ -18,8 +18,8 @@
 //    key range of an item is cut into splits (grid.x) and a split's tiles are
 //    dealt to the 4 waves, which stream K and V straight from the pages;
 //    partial (max, sum, O) go to scratch and fg_attn_combine merges them.
-//  * fg_attn_tile (prompt portions, 64 rows an item): K and V tiles are staged
-//    in LDS and shared by 4 waves of 16 rows each.
+//  * fg_attn_tile (prompt portions, up to 128 rows an item): K and V tiles are
+//    staged in LDS and shared by the workgroup's waves.
 //
 // Semantics as in attention.hip (fastgen/forward.py:176-258).
 #include "common.h"
@@ -439,32 +439,40 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
 }
 
 // ------------------------------------------------------------------- tile
-// grid n_items * n_kv, 256 threads: 4 waves of TILE_RB x 16 rows; an item has
-// at most TILE_ROWS / (H / KV) tokens.  The K and V tiles go through LDS in the order the
-// operands are read: K [4 key blocks][HD/8 chunks][16 keys][8], V [HD/16 dim
-// blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
-constexpr int TILE_RB = HD <= 128 ? 2 : 1;  // row blocks a wave holds (registers allow 2 up to head size 128)
-constexpr int TILE_ROWS = 64 * TILE_RB;     // query rows of an item
+// One workgroup per (item, kv head); an item has at most TILE_ROWS / (H / KV) tokens.  The K and
+// V tiles go through LDS in the order the operands are read: K [4 key blocks][HD/8 chunks]
+// [16 keys][8], V [HD/16 dim blocks][8 key chunks][16 dims][8 slots] (slots as in the permuted page).
+//
+// Up to head size 128: 8 waves and two tiles at a time.  Four row groups of 32 rows (two blocks of
+// 16 a wave, every K and V operand read serves both); the two waves of a row group take the even
+// and the odd tiles and merge their (max, sum, O) at the end.  The last rows of a long prompt see
+// every tile, one after the other: with two waves on them that chain is half as long, and a
+// compute unit holds one workgroup whose eight waves all work until its end.  Workgroups are
+// launched in the order of the items (most keys first), so short ones fill in behind long ones.
+// Above 128: 4 waves of 16 rows, one tile at a time (two tiles would not fit the 64 KB of LDS).
+constexpr bool TILE_PAIR = HD <= 128;
+constexpr int TILE_RB = TILE_PAIR ? 2 : 1;         // row blocks a wave holds
+constexpr int TILE_ROWS = 64 * TILE_RB;            // query rows of an item
+constexpr int TILE_THREADS = TILE_PAIR ? 512 : 256;
 
 template <bool PERM>
-__global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
+__global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_items, int n_heads,
-    int n_kv, int page_size, int page_shift, float scale, int window) {
-  // two tiles in LDS when they fit in 64 KB: tile i is read while tile i+1 is written and the loads
-  // of tile i+2 are in flight
-  constexpr int NBUF = HD <= 128 ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[NBUF][TILE * HD];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[NBUF][TILE * HD];
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
+    int page_size, int page_shift, float scale, int window) {
+  constexpr int NT = TILE_THREADS;
+  constexpr int NPT = TILE_PAIR ? 2 : 1;    // tiles a pass of the loop takes
+  // tiles in LDS: with pairs, one pair is read while the next is written (128 KB at head size 128, of
+  // the CU's 160 KB: the workgroup has the CU to itself anyway; measured 4 % faster than two slots)
+  constexpr int NSLOT = TILE_PAIR ? 4 : 1;
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[NSLOT][TILE * HD];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[NSLOT][TILE * HD];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
-  // (item, kv head) pairs in launch order: the first half ascending, the second half descending.
-  // Workgroups are handed out in order and a compute unit holds two, so where the items are the
-  // pieces of one prompt (work grows with the position) a late piece shares its unit with an early one.
-  const int n_pairs = gridDim.x, half = (n_pairs + 1) / 2;
-  const int pair = (int)blockIdx.x < half ? (int)blockIdx.x : n_pairs - 1 - ((int)blockIdx.x - half);
-  const int item = pair % n_items, kvh = pair / n_items;
+  const int rg = wave & 3;    // row group
+  const int par = wave >> 2;  // which tile of a pair this wave takes (0 when tiles come one at a time)
+  const int item = blockIdx.x / n_kv, kvh = blockIdx.x % n_kv;
   const int G = n_heads / n_kv;
   const Item it = load_item(items, item);
   const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
@@ -479,7 +487,7 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
   int w_all_hi = 0x7fffffff, w_all_lo = 0;  // keys in [w_all_lo, w_all_hi] are seen by all rows of the wave
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const int row = (wave * RB + rb) * 16 + r16;
+    const int row = (rg * RB + rb) * 16 + r16;
     const bool my_row = row < it.n_tok * G;
     const int my_tok = my_row ? row / G : 0, my_head = my_row ? row % G : 0;
     me[rb] = ItemRows{-1, 0};
@@ -516,13 +524,13 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
   const size_t head_elems = (size_t)page_size * HD;
   constexpr int KCH = HD / 8;                  // 16-byte chunks in a key
   constexpr int KTOT = TILE * KCH, VTOT = NDB * 8 * 16;  // chunks of a K tile, of a V tile
-  constexpr int KN = (KTOT + 255) / 256;       // K chunks a thread copies per tile
-  constexpr int VN = (VTOT + 255) / 256;       // V chunks a thread copies per tile
-  bf16x8 kreg[KN], vreg[VN];
-  // The next tile's chunks are fetched into registers while the current tile is computed from
-  // LDS.  Loads are never conditional: addresses are clamped into the item's key range, value
-  // slots outside it are masked, keys outside it give scores that the select discards.
-  auto fetch = [&](int k0) {
+  constexpr int KN = (KTOT + NT - 1) / NT;     // K chunks a thread copies per tile
+  constexpr int VN = (VTOT + NT - 1) / NT;     // V chunks a thread copies per tile
+  bf16x8 kreg[NPT][KN], vreg[NPT][VN];
+  // The next tiles' chunks are fetched into registers while the current ones are computed from
+  // LDS.  Loads are never conditional within a tile: addresses are clamped into the item's key
+  // range, value slots outside it are masked, keys outside it give scores that the select discards.
+  auto fetch = [&](int k0, bf16x8(&kr)[KN], bf16x8(&vr)[VN]) {
     if (PERM && (page_size & 63) == 0 && k0 >= first_min && k0 + TILE - 1 <= pos_last) {
       // The whole tile lies in one page and inside the key range: K's four 16-key blocks are 64*HD
       // contiguous elements in the order LDS wants them, V's eight key chunks are a contiguous run
@@ -533,30 +541,30 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
       const size_t v_block = (size_t)(page_size >> 3) * 128;  // elements of one block of 16 head dims
 #pragma unroll
       for (int j = 0; j < KN; ++j) {
-        const int w = min((int)threadIdx.x + 256 * j, KTOT - 1);
-        kreg[j] = *(const bf16x8*)(base_k + (size_t)w * 8);
+        const int w = min((int)threadIdx.x + NT * j, KTOT - 1);
+        kr[j] = *(const bf16x8*)(base_k + (size_t)w * 8);
       }
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
-        const int w = min((int)threadIdx.x + 256 * j, VTOT - 1);
-        vreg[j] = *(const bf16x8*)(base_v + (size_t)(w >> 7) * v_block + (size_t)(w & 127) * 8);
+        const int w = min((int)threadIdx.x + NT * j, VTOT - 1);
+        vr[j] = *(const bf16x8*)(base_v + (size_t)(w >> 7) * v_block + (size_t)(w & 127) * 8);
       }
       return;
     }
     // K: chunk (block kb, dims 8c.., key r) -> k_s[((kb*KCH + c)*16 + r)*8]; r fastest over threads
 #pragma unroll
     for (int j = 0; j < KN; ++j) {
-      const int w = min(threadIdx.x + 256 * j, KTOT - 1);  // beyond the tile: a copy that is not stored
+      const int w = min((int)threadIdx.x + NT * j, KTOT - 1);  // beyond the tile: a copy that is not stored
       const int r = w & 15, c = (w >> 4) % KCH, kb = (w >> 4) / KCH;
       const int key = min(max(k0 + 16 * kb + r, first_min), pos_last);
-      kreg[j] = *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
-                                 lay.k_off(pager.in_page(key), 8 * c));
+      kr[j] = *(const bf16x8*)(k_pages + ((size_t)pager.page_of(key) * n_kv + kvh) * head_elems +
+                               lay.k_off(pager.in_page(key), 8 * c));
     }
     // V: chunk (dim block db, key chunk kc = 4*ks + gg, dim r) -> v_s[((db*8 + kc)*16 + r)*8];
     // its slots are keys 32*ks + 4*gg + (0..3) and 16 more on
 #pragma unroll
     for (int j = 0; j < VN; ++j) {
-      const int w = min(threadIdx.x + 256 * j, VTOT - 1);
+      const int w = min((int)threadIdx.x + NT * j, VTOT - 1);
       const int r = w & 15, kc = (w >> 4) & 7, db = w >> 7;
       const int ka = k0 + 32 * (kc >> 2) + 4 * (kc & 3), kb2 = ka + 16;
       const bool in_a = ka + 3 >= first_min && ka <= pos_last;
@@ -580,17 +588,16 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
           v[4 + e] = hi[e];
         }
       }
-      vreg[j] = and_mask(v, slot_mask(ka, first_min, pos_last));
+      vr[j] = and_mask(v, slot_mask(ka, first_min, pos_last));
     }
   };
-  const int k_first = (first_min / TILE) * TILE;
-  auto stash = [&](int b) {
+  auto stash = [&](int b, const bf16x8(&kr)[KN], const bf16x8(&vr)[VN]) {
 #pragma unroll
     for (int j = 0; j < KN; ++j)
-      if (threadIdx.x + 256 * j < KTOT) *(bf16x8*)(k_lds[b] + (size_t)(threadIdx.x + 256 * j) * 8) = kreg[j];
+      if (threadIdx.x + NT * j < KTOT) *(bf16x8*)(k_lds[b] + (size_t)(threadIdx.x + NT * j) * 8) = kr[j];
 #pragma unroll
     for (int j = 0; j < VN; ++j)
-      if (threadIdx.x + 256 * j < VTOT) *(bf16x8*)(v_lds[b] + (size_t)(threadIdx.x + 256 * j) * 8) = vreg[j];
+      if (threadIdx.x + NT * j < VTOT) *(bf16x8*)(v_lds[b] + (size_t)(threadIdx.x + NT * j) * 8) = vr[j];
   };
   auto compute = [&](int k0, int b) {
     if (k0 > w_hi || k0 + TILE <= w_lo) return;  // nothing in this tile for this wave's rows
@@ -608,33 +615,77 @@ __global__ __launch_bounds__(256, HD <= 128 ? 2 : 1) void attn_tile_kernel(
     else
       attend_tile<false, RB, false>(k0, me, qop, scale * LOG2E, m, l, o, load_k, load_v);
   };
-  if (NBUF == 2) {
-    fetch(k_first);
-    stash(0);
-    if (k_first + TILE <= pos_last) fetch(k_first + TILE);
-    int b = 0;
-    for (int k0 = k_first; k0 <= pos_last; k0 += TILE, b ^= 1) {
-      __syncthreads();  // tile k0 is complete in buffer b; nobody reads buffer b^1 any more
-      if (k0 + TILE <= pos_last) stash(b ^ 1);
-      if (k0 + 2 * TILE <= pos_last) fetch(k0 + 2 * TILE);  // flies during this and the next tile's MFMAs
-      compute(k0, b);
+  const int k_first = (first_min / TILE) * TILE;
+  constexpr int STEP = NPT * TILE;  // keys per pass of the loop
+  auto fetch_pass = [&](int k0) {  // uniform conditions: a tile wholly beyond the range is not fetched
+    fetch(k0, kreg[0], vreg[0]);
+    if (NPT == 2 && k0 + TILE <= pos_last) fetch(k0 + TILE, kreg[NPT - 1], vreg[NPT - 1]);
+  };
+  auto stash_pass = [&](int k0, int s0) {
+    stash(s0, kreg[0], vreg[0]);
+    if (NPT == 2 && k0 + TILE <= pos_last) stash(s0 + NPT - 1, kreg[NPT - 1], vreg[NPT - 1]);
+  };
+  if (NSLOT == 2 * NPT) {
+    // pass i is read from its slots while pass i+1 is written to the other slots and the loads of
+    // pass i+2 are in flight: one barrier a pass
+    fetch_pass(k_first);
+    stash_pass(k_first, 0);
+    if (k_first + STEP <= pos_last) fetch_pass(k_first + STEP);
+    int s0 = 0;
+    for (int k0 = k_first; k0 <= pos_last; k0 += STEP, s0 ^= NPT) {
+      __syncthreads();  // pass k0 is complete in its slots; nobody reads the other slots any more
+      if (k0 + STEP <= pos_last) stash_pass(k0 + STEP, s0 ^ NPT);
+      if (k0 + 2 * STEP <= pos_last) fetch_pass(k0 + 2 * STEP);
+      const int mine = k0 + par * TILE;
+      if (mine <= pos_last) compute(mine, s0 + par);
     }
   } else {
-    fetch(k_first);
-    for (int k0 = k_first; k0 <= pos_last; k0 += TILE) {
+    fetch_pass(k_first);
+    for (int k0 = k_first; k0 <= pos_last; k0 += STEP) {
       __syncthreads();  // the previous tile is no longer read
-      stash(0);
+      stash_pass(k0, 0);
       __syncthreads();
-      if (k0 + TILE <= pos_last) fetch(k0 + TILE);  // flies during this tile's MFMAs
+      if (k0 + STEP <= pos_last) fetch_pass(k0 + STEP);  // flies during this tile's MFMAs
       compute(k0, 0);
     }
+  }
+  if (TILE_PAIR) {
+    // the odd tiles' wave hands its (max, sum, O) to the even tiles' wave of the same rows, one row
+    // block at a time, through the tiles' LDS; both waves hold the same rows in the same lanes
+    float* o_x = (float*)&k_lds[0][0];   // [4 row groups][NDB][64 lanes][4]
+    float* ml_x = (float*)&v_lds[0][0];  // [4 row groups][64 lanes][2]
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      __syncthreads();  // the tiles (or the previous row block) are no longer read
+      if (par == 1) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) *(f32x4*)(o_x + ((size_t)(rg * NDB + db) * FG_WAVE + lane) * 4) = o[rb][db];
+        ml_x[(rg * FG_WAVE + lane) * 2] = m[rb];
+        ml_x[(rg * FG_WAVE + lane) * 2 + 1] = l[rb];
+      }
+      __syncthreads();
+      if (par == 0) {
+        const float mo = ml_x[(rg * FG_WAVE + lane) * 2], lo = ml_x[(rg * FG_WAVE + lane) * 2 + 1];
+        const float M = fmaxf(m[rb], mo);
+        const float fs = m[rb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[rb] - M);
+        const float fo = mo == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mo - M);
+        l[rb] = fs * l[rb] + fo * lo;
+        m[rb] = M;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          const f32x4 other = *(const f32x4*)(o_x + ((size_t)(rg * NDB + db) * FG_WAVE + lane) * 4);
+          o[rb][db] = fs * o[rb][db] + fo * other;
+        }
+      }
+    }
+    if (par == 1) return;
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     float lsum = l[rb];
     lsum += __shfl_xor(lsum, 16, FG_WAVE);
     lsum += __shfl_xor(lsum, 32, FG_WAVE);
-    const int row = (wave * RB + rb) * 16 + r16;
+    const int row = (rg * RB + rb) * 16 + r16;
     if (row < it.n_tok * G) {
       bf16_t* orow = out + (size_t)(it.tok0 + row / G) * out_stride + (size_t)(kvh * G + row % G) * HD;
       const float inv = 1.f / lsum;
@@ -658,9 +709,9 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
       (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                        \
-  attn_tile_kernel<PERM><<<n_items * n_kv, 256, 0, stream>>>(                                               \
+  attn_tile_kernel<PERM><<<n_items * n_kv, TILE_THREADS, 0, stream>>>(                                      \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
-      block_table, bt_stride, items, n_items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
+      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
   if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
 #undef LAUNCH
   return fg_launch_status();
