@@ -367,21 +367,29 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
   __shared__ float f_s[COMBINE_MAX_SPLITS];  // weight of each split's partial output: 2^(m_s - M) / L
   const int r = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z, d = threadIdx.x;
   const int G = n_heads / n_kv;
-  const Item it = load_item(items, item);
-  if (r >= it.n_tok * G) return;  // the whole workgroup
+  // where the partial results lie depends on the indices alone: their loads go out together with
+  // the item's, one round trip for all of them
   const size_t row0 = (((size_t)item * n_kv + kvh) * n_splits) * 16 + r;
+  const int dc = min(d, HD - 1);
+  float first[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) first[u] = part_o[(row0 + (size_t)min(u, n_splits - 1) * 16) * HD + dc];
+  constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
+  float ms[PER], ls[PER];
   if (threadIdx.x < FG_WAVE) {
-    constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
-    float ms[PER], ls[PER];
-    float M = -INFINITY;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int sp = threadIdx.x + j * FG_WAVE;
       const float2 ml = *(const float2*)(part_ml + (row0 + (size_t)min(sp, n_splits - 1) * 16) * 2);
       ms[j] = sp < n_splits ? ml.x : -INFINITY;  // maxima are in base 2
       ls[j] = ml.y;
-      M = fmaxf(M, ms[j]);
     }
+  }
+  const Item it = load_item(items, item);
+  if (threadIdx.x < FG_WAVE) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) M = fmaxf(M, ms[j]);
     M = wave_max(M);
     float L = 0.f;
 #pragma unroll
@@ -395,9 +403,11 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     for (int j = 0; j < PER; ++j) f_s[threadIdx.x + j * FG_WAVE] = ms[j] * inv;
   }
   __syncthreads();
-  if (d >= HD) return;
+  if (d >= HD || r >= it.n_tok * G) return;  // (a row beyond the item: its partial results are never written)
   float O = 0.f;
-  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+#pragma unroll
+  for (int u = 0; u < 8; ++u) O += (u < n_splits ? f_s[u] : 0.f) * first[u];
+  for (int s0 = 8; s0 < n_splits; s0 += 8) {
     float v[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) v[u] = part_o[(row0 + (size_t)min(s0 + u, n_splits - 1) * 16) * HD + d];

@@ -92,45 +92,55 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   float* hrow = h + src * dim;
   const TA* drow = delta ? delta + src * dim : nullptr;
-  float v[NIT][8];
+  // Every load of the row is issued before anything is added (the kernel is a chain of memory
+  // round trips: as few of them as possible).  Loads are never conditional: a thread whose share
+  // lies beyond the row reads the row's last 8 elements and stores nothing.
+  int e[NIT], ec[NIT];
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
-    if (e < dim) load8<float>(hrow + e, v[it]);
+    e[it] = (threadIdx.x + it * ROWS_THREADS) * 8;
+    ec[it] = min(e[it], dim - 8);
   }
-  if (drow || parts) {
+  float v[NIT][8], wv[NIT][8];
 #pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
-      if (e < dim) {
-        float d[8];
-        if (drow) {
-          load8<TA>(drow + e, d);
+  for (int it = 0; it < NIT; ++it) load8<float>(hrow + ec[it], v[it]);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) v[it][i] += d[i];
-        }
-        if (parts) {
-          // eight partial results at a time, all loads issued before the first is added
-          for (int p0 = 0; p0 < n_parts; p0 += 8) {
-            float dp[8][8];
+  for (int it = 0; it < NIT; ++it) load8<TW>(w + ec[it], wv[it]);
+  if (drow) {
+    float d[NIT][8];
 #pragma unroll
-            for (int p = 0; p < 8; ++p)
-              load8<float>(parts + (size_t)min(p0 + p, n_parts - 1) * part_stride + src * dim + e, dp[p]);
+    for (int it = 0; it < NIT; ++it) load8<TA>(drow + ec[it], d[it]);
 #pragma unroll
-            for (int p = 0; p < 8; ++p)
+    for (int it = 0; it < NIT; ++it)
 #pragma unroll
-              for (int i = 0; i < 8; ++i) v[it][i] += p0 + p < n_parts ? dp[p][i] : 0.f;
-          }
-        }
-        if (!rows) store8<float>(hrow + e, v[it]);
-      }
+      for (int i = 0; i < 8; ++i) v[it][i] += d[it][i];
+  }
+  if (parts) {
+    constexpr int PB = NIT <= 2 ? 8 : 4;  // partial results whose loads are in flight together
+    for (int p0 = 0; p0 < n_parts; p0 += PB) {
+      float dp[NIT][PB][8];
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int p = 0; p < PB; ++p)
+          load8<float>(parts + (size_t)min(p0 + p, n_parts - 1) * part_stride + src * dim + ec[it], dp[it][p]);
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int p = 0; p < PB; ++p)  // in order of the partial results
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v[it][i] += p0 + p < n_parts ? dp[it][p][i] : 0.f;
     }
+  }
+  if ((drow || parts) && !rows) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+      if (e[it] < dim) store8<float>(hrow + e[it], v[it]);
   }
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
-    if (e < dim) {
+    if (e[it] < dim) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) ss += v[it][i] * v[it][i];
     }
@@ -140,13 +150,11 @@ __global__ __launch_bounds__(ROWS_THREADS) void add_rmsnorm_vec_kernel(
   TA* orow = out + (size_t)r * dim;
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
-    const int e = (threadIdx.x + it * ROWS_THREADS) * 8;
-    if (e < dim) {
-      float wv[8], o[8];
-      load8<TW>(w + e, wv);
+    if (e[it] < dim) {
+      float o[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o[i] = v[it][i] * rstd * wv[i];
-      store8<TA>(orow + e, o);
+      for (int i = 0; i < 8; ++i) o[i] = v[it][i] * rstd * wv[it][i];
+      store8<TA>(orow + e[it], o);
     }
   }
 }
