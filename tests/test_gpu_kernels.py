@@ -464,6 +464,33 @@ def test_top_p_keeps_the_reference_set(ops):
         assert seen[likely].all()  # every kept token that should show up does
 
 
+@pytest.mark.parametrize("p", [0.04, 0.3, 0.9])
+def test_top_p_draws_follow_the_kept_distribution(ops, p):
+    """The draws are distributed as the kept tokens' probabilities, renormalised
+    (the reference draws with multinomial from the un-renormalised rest).  The
+    smallest p makes most first draws miss the kept set, so that the exact
+    search for the kept set's edge is taken as well."""
+    V, n = 1031, 30000
+    torch.manual_seed(14)
+    row = torch.randn(V) * 2
+    probs = torch.softmax(row / 0.9, -1)
+    keep = plain_top_p_keep(probs[None], p)[0]
+    logits = row[None].expand(n, V).contiguous().to(DEV)
+    got = ops.sample(logits, torch.full((n,), 0.9, device=DEV), torch.full((n,), p, device=DEV),
+                     torch.full((n,), 99, dtype=torch.int64, device=DEV),
+                     torch.arange(n, dtype=torch.int64, device=DEV)).cpu().long()
+    assert keep[got].all()
+    want = probs * keep / (probs * keep).sum()
+    counts = torch.bincount(got, minlength=V).float()
+    big = n * want >= 10  # cells with enough expected draws; the others as one cell
+    obs = torch.cat([counts[big], counts[~big].sum()[None]])
+    exp = torch.cat([n * want[big], (n * want[~big]).sum()[None]])
+    ok = exp > 0
+    chi2 = float(((obs[ok] - exp[ok]) ** 2 / exp[ok]).sum())
+    dof = int(ok.sum()) - 1
+    assert chi2 < dof + 6 * math.sqrt(2 * max(dof, 1)) + 10, (chi2, dof)
+
+
 def test_logprob(ops):
     torch.manual_seed(13)
     logits = torch.randn(4, 1000) * 5
