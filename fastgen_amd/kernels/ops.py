@@ -267,7 +267,8 @@ def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int =
     position of the first token): items of at most 16 rows for the split
     kernel (decoded tokens and very short portions) and items of at most
     ``tile_rows`` rows for the tile kernel, those with the most keys first (the
-    kernel starts them in that order and pairs the first with the last).
+    kernel's workgroups start in that order, so short items fill in behind long
+    ones).
     """
     small, big = [], []
     per_tile = max(1, tile_rows // group_size)
