@@ -32,10 +32,16 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
         gate, up = tensors[self._name("gate_proj.weight")], tensors[self._name("up_proj.weight")]
-        if self.hidden_dim % 8:
-            raise ValueError(f"{self.prefix}: hidden_dim={self.hidden_dim} must be a multiple of 8")
+        down = tensors[self._name("down_proj.weight")]
+        pad = -self.hidden_dim % 8
+        if pad:
+            # the kernels work on groups of 8 channels: channels of zero weights are added, whose
+            # activation silu(0) * 0 = 0 meets zero columns of the down projection
+            gate = torch.cat([gate, gate.new_zeros(pad, self.dim)])
+            up = torch.cat([up, up.new_zeros(pad, self.dim)])
+            down = torch.cat([down, down.new_zeros(self.dim, pad)], dim=1)
         self.w_gate_up = place(ops.interleave_gate_up(gate, up), MATRIX, dtype, device)
-        self.w_down = place(tensors[self._name("down_proj.weight")], MATRIX, dtype, device)
+        self.w_down = place(down, MATRIX, dtype, device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if wide_ok(x, self.w_gate_up):

@@ -28,12 +28,13 @@ def _close(got, want, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_norm_feed_forward_embedding_head_alone(dtype):
+@pytest.mark.parametrize("F", [200, 77])  # 77: not a multiple of the 8 channels the kernels group
+def test_norm_feed_forward_embedding_head_alone(dtype, F):
     from fastgen_amd.config import PartSpec
     from fastgen_amd.parts import build_part
 
     torch.manual_seed(0)
-    D, F, V, T = 72, 200, 131, 9
+    D, V, T = 72, 131, 9
     norm = build_part("norm", PartSpec("rmsnorm", "n", dict(dim=D, eps=1e-3)))
     w = 1 + 0.1 * torch.randn(D)
     norm.load({"n.weight": w}, dtype, DEV)
