@@ -71,20 +71,28 @@ class StepContext:
 
 
 def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: Optional[int] = None,
-                 table_width: Optional[int] = None):
+                 table_width: Optional[int] = None, pad_to: Optional[int] = None):
     """Host side of :func:`build_context`: every int32 vector of the step in
     one numpy buffer, and where each lies in it.  With ``table_width`` the block
     tables have that many columns whatever the requests hold, so that steps of
-    the same batch shape have the same layout."""
-    B = len(entries)
+    the same batch shape have the same layout.  With ``pad_to`` the batch is
+    filled up to that many sequences with stand-ins of one token at position 0
+    that write nothing to the cache (slot -1) and own no page (their block
+    table rows name page 0, which they only read): a captured step of
+    ``pad_to`` sequences then serves any smaller batch; the stand-ins' logits
+    are the last rows and mean nothing."""
+    n_real = len(entries)
     q_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
-    if B == 0 or (q_lens <= 0).any():
+    if n_real == 0 or (q_lens <= 0).any():
         raise ValueError("a step needs at least one entry and every entry at least one token")
-    n_cached = np.array([cache.length(e.rid) for e in entries], dtype=np.int32)
+    n_pad = max(0, (pad_to or 0) - n_real)
+    B = n_real + n_pad
+    q_lens = np.concatenate([q_lens, np.ones(n_pad, dtype=np.int32)])
+    n_cached = np.array([cache.length(e.rid) for e in entries] + [0] * n_pad, dtype=np.int32)
     q_start = np.zeros(B + 1, dtype=np.int32)
     np.cumsum(q_lens, out=q_start[1:])
     T = int(q_start[-1])
-    tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+    tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries] + [np.zeros(n_pad, dtype=np.int64)])
     if (tokens < 0).any() or (vocab_size is not None and (tokens >= vocab_size).any()):
         raise ValueError(f"token id outside [0, {vocab_size})")
     seq_of_token = np.repeat(np.arange(B, dtype=np.int32), q_lens)
@@ -95,7 +103,8 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
             if not 0 <= w < q_lens[b]:
                 raise ValueError(f"request {e.rid!r}: wanted place {w} is outside its {q_lens[b]} tokens")
             out_rows.append(int(q_start[b]) + int(w))
-    slot_ids = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
+    out_rows += [int(q_start[b]) for b in range(n_real, B)]
+    slot_ids = np.array([cache.slot(e.rid) for e in entries] + [0] * n_pad, dtype=np.int32)
 
     # one record per sequence (sequence, first flat token, tokens, first position): the items of the
     # attention kernels when every sequence brings so few tokens that it is one item; first in the
@@ -111,7 +120,7 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
                 raise ValueError(f"a request holds {width} pages, the fixed table width is {table_width}")
             width = table_width
         tbl = np.zeros((B, max(1, width)), dtype=np.int32)
-        slots = np.empty(T, dtype=np.int32)
+        slots = np.full(T, -1, dtype=np.int32)
         for b, e in enumerate(entries):
             row = cache.pages_of(e.rid, g)
             tbl[b, : len(row)] = row

@@ -75,7 +75,7 @@ class Engine:
     def step(self) -> List[Request]:
         """One step of the model over what the scheduler picks; the requests
         that ended with it."""
-        n_run = self.scheduler.plan_decode_run(self.sync_freq) if self.runner.use_graphs else 0
+        n_run = self.scheduler.plan_decode_run(self.sync_freq) if self.runner.can_graph(len(self.scheduler.running)) else 0
         if n_run:
             return self._decode_run(n_run)
         plan = self.scheduler.plan()

@@ -22,20 +22,31 @@ from .context import StepContext, StepEntry, build_context, context_from_packed,
 from .model import Model
 
 
+def graph_capacity_for(n: int) -> int:
+    """The number of sequences of the captured step that serves a decode batch
+    of ``n``: every size up to 16, then steps of 8, 16 and 32, so that a few
+    dozen captures cover hundreds of batch sizes (the reference spaces its 16
+    graphs likewise and pads, ``fastgen/generate.py:296-352``)."""
+    if n <= 16:
+        return n
+    step = 8 if n <= 64 else 16 if n <= 128 else 32
+    return -(-n // step) * step
+
+
 class _DecodeGraph:
     """One captured decode step for a fixed number of sequences.
 
     The step's int32 vectors live in a device buffer of fixed layout (block
     tables as wide as a request can get); a replay copies the new values in
     and runs the captured kernels, which read lengths and pages from that
-    buffer.  (The reference captures 16 such graphs at spaced batch sizes and
-    pads, ``fastgen/generate.py:296-352``; here a graph is captured for each
-    batch size when it first occurs.)
+    buffer.  A smaller batch is filled up with stand-in sequences that write
+    nothing; a graph is captured when a batch of its capacity first occurs.
     """
 
     def __init__(self, runner: "ModelRunner", entries: Sequence[StepEntry]) -> None:
         model, cache = runner.model, runner.cache
-        packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, runner.table_width)
+        self.capacity = graph_capacity_for(len(entries))
+        packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, runner.table_width, self.capacity)
         self.layout = (tuple(int(o) for o in offs), tuple(shapes))
         # a ring of pinned staging buffers: the host may run several steps ahead of the device
         self.staging = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(runner.run_ahead)]
@@ -65,8 +76,9 @@ class _DecodeGraph:
         """Copy the step's vectors in and run the captured step.  With
         ``tokens_on_device`` (int32 ``[B]``) the tokens come from there, not from
         ``entries``: the step before sampled them and the host has not seen them."""
+        n = len(entries)
         packed, offs, shapes, host = pack_context(entries, runner.cache, None if tokens_on_device is not None
-                                                  else runner.model.vocab_size, runner.table_width)
+                                                  else runner.model.vocab_size, runner.table_width, self.capacity)
         if (tuple(int(o) for o in offs), tuple(shapes)) != self.layout:
             raise RuntimeError("decode graph: the step's layout differs from the captured one")
         i = self.turn = (self.turn + 1) % len(self.staging)
@@ -75,9 +87,9 @@ class _DecodeGraph:
         self.packed.copy_(self.staging[i], non_blocking=True)
         self.copied[i].record()
         if tokens_on_device is not None:
-            self.ctx.tokens.copy_(tokens_on_device)
+            self.ctx.tokens[:n].copy_(tokens_on_device)
         self.graph.replay()
-        return self.logits
+        return self.logits[:n]
 
 
 class ModelRunner:
@@ -109,7 +121,7 @@ class ModelRunner:
         self.table_width = max(1, max(pages, default=1))
         self.graphs: Dict[int, _DecodeGraph] = {}
         self.graph_pool = None
-        self.max_graphs = 32
+        self.max_graphs = 64
         self.run_ahead = 16  # steps the host may prepare before the device has run them
 
     # ------------------------------------------------------------ requests
@@ -156,7 +168,18 @@ class ModelRunner:
         """One token a request, its logits wanted, every request already live."""
         return bool(entries) and all(
             len(e.tokens) == 1 and list(e.want) == [0] and self.cache.is_live(e.rid) for e in entries
-        ) and (len(entries) in self.graphs or len(self.graphs) < self.max_graphs)
+        ) and self.can_graph(len(entries))
+
+    def can_graph(self, n: int) -> bool:
+        """Whether a decode batch of ``n`` has, or may still get, a captured step."""
+        return self.use_graphs and (graph_capacity_for(n) in self.graphs or len(self.graphs) < self.max_graphs)
+
+    def _graph_for(self, entries: Sequence[StepEntry]) -> _DecodeGraph:
+        cap = graph_capacity_for(len(entries))
+        g = self.graphs.get(cap)
+        if g is None:
+            g = self.graphs[cap] = _DecodeGraph(self, entries)
+        return g
 
     def decode_run(self, entries: Sequence[StepEntry], n_steps: int, sample) -> torch.Tensor:
         """``n_steps`` decode steps of the same requests without the host seeing
@@ -171,9 +194,7 @@ class ModelRunner:
         n_steps = min(n_steps, self.run_ahead - 1)
         for e in entries:
             self.cache.reserve(e.rid, n_steps)
-        g = self.graphs.get(len(entries))
-        if g is None:
-            g = self.graphs[len(entries)] = _DecodeGraph(self, entries)
+        g = self._graph_for(entries)
         out = torch.empty((n_steps, len(entries)), dtype=torch.int32, device=self.model.device)
         for s in range(n_steps):
             logits = g.replay(self, entries, out[s - 1] if s else None)
@@ -187,8 +208,5 @@ class ModelRunner:
             raise ValueError("a request appears twice in one step")
         for e in entries:
             self.cache.reserve(e.rid, 1)
-        g = self.graphs.get(len(entries))
-        if g is None:
-            g = self.graphs[len(entries)] = _DecodeGraph(self, entries)
-            # the capture ran the step's kernels only as a recording: replay it for this step's result
-        return g.replay(self, entries)
+        # (a capture runs the step's kernels only as a recording: the replay gives this step's result)
+        return self._graph_for(entries).replay(self, entries)
