@@ -2,6 +2,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py --workload serve        # continuous batching, see serve_workload()
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -35,6 +36,57 @@ CONTEXT_LEN = 8192  # capacity per request
 PAGE = 64
 
 
+LLAMA_3B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=3072, intermediate_size=8192, num_hidden_layers=28,
+    num_attention_heads=24, num_key_value_heads=8, rms_norm_eps=1e-5, vocab_size=128256, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True, max_position_embeddings=131072,
+)
+
+
+def serve_workload(n_requests: int = 256) -> int:
+    """Continuous batching at the Llama 3.2 3B shape (random bfloat16 weights): ``n_requests`` requests
+    arrive at once, prompts of 128..4096 uniform random ids, 32..512 greedy tokens each, at most 256 live,
+    a budget of 2,048 tokens a step (prompt portions beside decoded tokens).  One JSON line: generated
+    tokens a second over the whole run, prompt processing included."""
+    import random
+
+    import torch
+
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    rng = random.Random(3)
+    plens = [rng.randint(128, 4096) for _ in range(n_requests)]
+    olens = [rng.randint(32, 512) for _ in range(n_requests)]
+    max_batch = min(256, n_requests)
+    engine = Engine.from_config(LLAMA_3B, seed=3, dtype=torch.bfloat16, page_size=PAGE, max_tokens=max_batch * 4672,
+                                max_batch=max_batch, max_step_tokens=2048)
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, LLAMA_3B["vocab_size"], (n,), generator=g).tolist() for n in plens]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for p, o in zip(prompts, olens):
+        engine.add_request(p, SamplingParams(temperature=0.0, max_new_tokens=o))
+    n_done, last = 0, t0
+    while engine.has_work():
+        n_done += len(engine.step())
+        if time.perf_counter() - last > 20:
+            last = time.perf_counter()
+            print(f"[bench] {n_done}/{n_requests} requests done", file=sys.stderr, flush=True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    print(json.dumps({
+        "metric": "generated tok/s, continuous batching", "value": round(sum(olens) / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": "llama-3.2-3b-shape-random", "requests": n_requests, "prompt_tokens": sum(plens),
+                   "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": 2048, "page_size": PAGE,
+                   "engine_steps": engine.n_steps, "preemptions": engine.scheduler.n_preemptions},
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -44,10 +96,14 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--workload", choices=["decode", "serve"], default="decode",
+                    help="decode (default): the step benchmark; serve: continuous batching of 256 requests")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported", flush=True)
         return 2
+    if a.workload == "serve":
+        return serve_workload()
 
     import torch
 
