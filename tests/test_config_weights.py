@@ -187,3 +187,16 @@ def test_dtype_policy():
     assert place(torch.randn(4), VECTOR, torch.bfloat16, "cpu").dtype == torch.float32  # stored in 32-bit: stays
     assert place(torch.randn(4).bfloat16(), VECTOR, torch.bfloat16, "cpu").dtype == torch.bfloat16
     assert place(torch.arange(4), TABLE_INT, torch.bfloat16, "cpu").dtype == torch.int32
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py runs on one GPU: for more it says so in one line and exits with 2."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parent.parent / "bench.py"
+    r = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
+
