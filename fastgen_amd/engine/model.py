@@ -114,6 +114,10 @@ class Model:
                 out[i] = need
         return out
 
+    def capturable(self) -> bool:
+        """Whether every part's forward may be recorded into a HIP graph."""
+        return all(getattr(p, "capturable", True) for p in self.parts.all_parts)
+
     def weight_bytes(self) -> int:
         seen, total = set(), 0
         for p in self.parts.all_parts:

@@ -117,7 +117,8 @@ class ModelRunner:
         # decode graphs: FG_NO_GRAPHS=1 switches them off (the reference: FG_NO_CUDA_GRAPHS)
         # a mixer with state of its own is stepped eagerly: the warm-up run before a capture would
         # advance its state twice
-        self.use_graphs = os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and not model.state_needs()
+        self.use_graphs = (os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and not model.state_needs()
+                           and model.capturable())
         self.table_width = max(1, max(pages, default=1))
         self.graphs: Dict[int, _DecodeGraph] = {}
         self.graph_pool = None

@@ -76,7 +76,15 @@ class LayerStore:
 
 
 class Part:
-    """Base of every part: declares its tensors and takes them when loaded."""
+    """Base of every part: declares its tensors and takes them when loaded.
+
+    ``capturable``: whether ``forward`` may be recorded into a HIP graph, that
+    is, whether it launches the same kernels with the same arguments whatever
+    the values on the device are.  A part that looks at device data on the
+    host (shapes that depend on the data) sets it to False; a model with such
+    a part is always stepped eagerly."""
+
+    capturable: bool = True
 
     def __init__(self, spec: PartSpec) -> None:
         self.spec = spec

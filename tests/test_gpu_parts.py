@@ -152,23 +152,26 @@ class _HybridArch:
         for i, l in enumerate(a["layers"]):
             p = f"blocks.{i}"
             if l["mixer"] == "attention":
-                pos = PartSpec("rope", options=dict(head_dim=l["hd"], rotary_dim=l.get("rot", l["hd"]), theta=a["theta"]))
+                pos = PartSpec(l.get("pos", "rope"), options=dict(head_dim=l["hd"], rotary_dim=l.get("rot", l["hd"]),
+                                                                  theta=a["theta"], **l.get("pos_options", {})))
                 mixer = PartSpec("attention", f"{p}.attn", dict(dim=D, n_heads=l["H"], n_kv_heads=l["KV"],
                                                                head_dim=l["hd"], scale=l["hd"] ** -0.5,
                                                                window=l.get("window"), position=pos))
             else:
                 mixer = PartSpec(l["mixer"], f"{p}.mix", dict(dim=D, decay=l["decay"]))
-            layers.append(LayerSpec(mixer, PartSpec("swiglu", f"{p}.ffn", dict(dim=D, hidden_dim=l["F"])),
-                                    norm(f"{p}.n1"), norm(f"{p}.n2")))
+            ffn = PartSpec(l.get("ffn", "swiglu"), f"{p}.ffn", dict(dim=D, hidden_dim=l["F"], **l.get("ffn_options", {})))
+            layers.append(LayerSpec(mixer, ffn, norm(f"{p}.n1"), norm(f"{p}.n2")))
         order = tuple(RunEntry(o[0], o[1]) for o in a["order"])
         return ModelLayout(D, a["vocab"], PartSpec("embedding", "emb", dict(vocab_size=a["vocab"], dim=D)),
                            tuple(layers), order, norm("final"),
                            PartSpec("lm_head", "head", dict(vocab_size=a["vocab"], dim=D, tied_to=None)))
 
 
-def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32):
+def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32, ffns=None, positions=None):
     """Plain whole-sequence forward of the hybrid model; attention entries
-    that read another entry's cache use that entry's rotated k and v."""
+    that read another entry's cache use that entry's rotated k and v.
+    ``mixers`` / ``ffns`` / ``positions``: plain functions of the toy parts
+    by kind."""
     T = len(tokens)
     w = {k: v.to(dtype) for k, v in w.items()}
     h = w["emb.weight"][torch.tensor(tokens)]
@@ -181,6 +184,8 @@ def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32):
             f = plain_rope_frequencies(rot, a["theta"])
 
             def rope(t, nh):
+                if l.get("pos", "rope") != "rope":
+                    return positions[l["pos"]](t, l, a)
                 perm = plain_rope_shuffle(torch.eye(nh * rot, dtype=dtype), nh)
                 tr = t[..., :rot].reshape(T, nh * rot) @ perm.T
                 tr = plain_rope_interleaved(tr.view(T, nh, rot), torch.arange(T), f)
@@ -198,6 +203,9 @@ def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32):
             m = mixers[l["mixer"]](x, w, p, l)
         h = h + m
         x = plain_rmsnorm(h, w[f"{p}.n2.weight"], a["eps"])
+        if l.get("ffn", "swiglu") != "swiglu":
+            h = h + ffns[l["ffn"]](x, w, p, l)
+            continue
         h = h + plain_swiglu(x, w[f"{p}.ffn.gate_proj.weight"], w[f"{p}.ffn.up_proj.weight"],
                              w[f"{p}.ffn.down_proj.weight"])
     return (plain_rmsnorm(h, w["final.weight"], a["eps"]) @ w["head.weight"].T).float()
@@ -321,3 +329,110 @@ def test_toy_mixer_with_state_of_its_own(tmp_path, hybrid_arch):
         assert runner.cache.free_slots() == 2
     finally:
         unregister_part("mixer", "toy_ema")
+
+
+# ------------------------------------- a toy feed-forward with routing, a toy position encoding
+def _register_toy_ffn_and_position():
+    from fastgen_amd.parts import FeedForward, PositionEncoding, TensorSpec, place, register_part
+
+    class ToyRouted(FeedForward):
+        """Each row goes to the expert its router row scores highest (router in
+        fp32), weighted by that expert's softmax probability; an expert is a
+        SwiGLU of its own.  Plain torch on the device: a toy.  It asks the
+        device which rows went where, so its steps cannot be captured."""
+
+        capturable = False
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            o = spec.options
+            self.dim, self.hidden, self.n_experts = o["dim"], o["hidden_dim"], o["n_experts"]
+
+        def tensor_specs(self):
+            specs = [TensorSpec(self._name("router.weight"), (self.n_experts, self.dim))]
+            for e in range(self.n_experts):
+                specs += [TensorSpec(self._name(f"experts.{e}.gate_proj.weight"), (self.hidden, self.dim)),
+                          TensorSpec(self._name(f"experts.{e}.up_proj.weight"), (self.hidden, self.dim)),
+                          TensorSpec(self._name(f"experts.{e}.down_proj.weight"), (self.dim, self.hidden))]
+            return specs
+
+        def load(self, tensors, dtype, device):
+            self.router = tensors[self._name("router.weight")].to(device=device, dtype=torch.float32)
+            self.experts = [tuple(place(tensors[self._name(f"experts.{e}.{k}_proj.weight")], "matrix", dtype, device)
+                                  for k in ("gate", "up", "down")) for e in range(self.n_experts)]
+
+        def forward(self, x):
+            probs = torch.softmax(x.float() @ self.router.T, -1)
+            weight, choice = probs.max(-1)
+            out = torch.zeros_like(x)
+            for e, (wg, wu, wd) in enumerate(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    xe = x[rows]
+                    g = xe @ wg.T
+                    y = ((g * torch.sigmoid(g)) * (xe @ wu.T)) @ wd.T
+                    out[rows] = (y.float() * weight[rows, None]).to(x.dtype)
+            return out
+
+    class ToyLinearRope(PositionEncoding):
+        """Rotation of interleaved pairs as stored (no reordering of rows), all
+        frequencies divided by a factor."""
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            o = spec.options
+            self.rotary_dim, self.theta, self.factor = int(o["rotary_dim"]), float(o["theta"]), float(o["factor"])
+
+        def frequencies(self):
+            return plain_rope_frequencies(self.rotary_dim, self.theta) / self.factor
+
+    register_part("feed_forward", "toy_routed", ToyRouted, replace=True)
+    register_part("position", "toy_linear", ToyLinearRope, replace=True)
+
+
+def _plain_toy_routed(x, w, p, l):
+    probs = torch.softmax(x.float() @ w[f"{p}.ffn.router.weight"].float().T, -1)
+    weight, choice = probs.max(-1)
+    out = torch.zeros_like(x)
+    for t in range(x.shape[0]):
+        e = int(choice[t])
+        y = plain_swiglu(x[t : t + 1], w[f"{p}.ffn.experts.{e}.gate_proj.weight"], w[f"{p}.ffn.experts.{e}.up_proj.weight"],
+                         w[f"{p}.ffn.experts.{e}.down_proj.weight"])
+        out[t] = y[0] * weight[t]
+    return out
+
+
+def _plain_toy_linear_rope(t, l, a):
+    f = plain_rope_frequencies(l["hd"], a["theta"]) / l["pos_options"]["factor"]
+    return plain_rope_interleaved(t, torch.arange(t.shape[0]), f)
+
+
+def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, hybrid_arch):
+    """A feed-forward that routes rows to experts and a rotary scheme of its
+    own, both defined here and registered: built, loaded and stepped without a
+    change to the framework, under cuts and batches."""
+    from fastgen_amd.engine import Model, ModelRunner
+    from fastgen_amd.parts import unregister_part
+
+    _register_toy_ffn_and_position()
+    try:
+        args = dict(dim=64, vocab=101, eps=1e-5, theta=1000.0, layers=[
+            dict(mixer="attention", H=4, KV=2, hd=16, pos="toy_linear", pos_options=dict(factor=4.0), F=40,
+                 ffn="toy_routed", ffn_options=dict(n_experts=3)),
+            dict(mixer="attention", H=2, KV=1, hd=32, F=96),
+        ], order=[(0, None), (1, None)])
+        folder, w = _hybrid_case(tmp_path, args, seed=6)
+        model = Model.from_folder(folder, torch.float32, DEV)
+        runner = ModelRunner(model, page_size=16, max_tokens=512, max_requests=4)
+        assert not runner.use_graphs
+        lengths = {"a": 45, "b": 18, "c": 3}
+        g = torch.Generator().manual_seed(8)
+        toks = {r: torch.randint(0, 101, (n,), generator=g).tolist() for r, n in lengths.items()}
+        want = {r: _plain_hybrid(w, args, t, {}, ffns={"toy_routed": _plain_toy_routed},
+                                 positions={"toy_linear": _plain_toy_linear_rope}) for r, t in toks.items()}
+        for tr in (traces.whole(lengths), traces.chunks(lengths), traces.mixed(lengths, seed=5)):
+            assert_close(run_trace(runner, tr, toks), want, torch.float32, None, "toy ffn / position")
+    finally:
+        unregister_part("feed_forward", "toy_routed")
+        unregister_part("position", "toy_linear")
+
