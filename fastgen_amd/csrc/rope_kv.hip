@@ -116,9 +116,8 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
   const size_t head_elems = (size_t)page_size * hd;
   const int cph = hd / 8;  // chunks per head
   const int n_rot = (n_heads + (write_kv ? n_kv : 0)) * cph;
-  const int n_v = slot >= 0 ? n_kv * cph : 0;
-  for (int w = threadIdx.x; w < n_rot + n_v; w += ROPE_THREADS) {
-    if (w < n_rot) {
+  for (int w = threadIdx.x; w < n_rot; w += ROPE_THREADS) {
+    {
       const int head = w / cph, c = w % cph;
       if (head >= n_heads && slot < 0) continue;
       T* x = row + (size_t)head * hd + 8 * c;
@@ -148,12 +147,15 @@ __global__ __launch_bounds__(ROPE_THREADS) void rope_kv_write_vec_kernel(
         store8<T>(x, v);
       else
         store8<T>(k_pages + ((size_t)page * n_kv + (head - n_heads)) * head_elems + lay.k_off(off, 8 * c), v);
-    } else {
-      const int e = w - n_rot, kvh = e / cph, c = e % cph;
-      const T* src = row + (size_t)(n_heads + n_kv + kvh) * hd + 8 * c;
-      T* dst = v_pages + ((size_t)page * n_kv + kvh) * head_elems;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) dst[lay.v_off(off, 8 * c + i)] = src[i];
+    }
+  }
+  if (slot >= 0) {
+    // v: one element a thread, consecutive threads consecutive head dims: in the transposed page
+    // these lie 16 bytes apart, so a wave's store stays within a few cache lines
+    const T* v = row + (size_t)(n_heads + n_kv) * hd;
+    for (int e = threadIdx.x; e < n_kv * hd; e += ROPE_THREADS) {
+      const int kvh = e / hd, d = e % hd;
+      v_pages[((size_t)page * n_kv + kvh) * head_elems + lay.v_off(off, d)] = v[e];
     }
   }
 }
