@@ -3,7 +3,7 @@
 (``fastgen/generate.py:30-76, 138-173, 405-475``), with the same names and
 meanings of options where the reference has them.
 
-    fg = Fastgen.build(model_dir, GenArgs(max_batch=8, max_gen=64))
+    fg = Fastgen.build(HfLoader(model_dir), GenArgs(max_batch=8, max_gen=64))     # or the folder itself
     q = queue.Queue(); q.put(Packet(thread_id=0, tokens=[1, 2, 3])); q.put(None)
     for pkt in fg.generate(q):
         print(pkt.thread_id, pkt.tokens)
@@ -71,19 +71,55 @@ def cache_tokens_for_budget(model: Model, gen_args: GenArgs, bytes_per_token: in
     return -(-tokens // gen_args.cache_block) * gen_args.cache_block
 
 
+class HfLoader:
+    """A model folder in the Hugging Face layout: ``config.json``,
+    ``model.safetensors`` (or shards with an index) and, optionally,
+    ``tokenizer.json`` (``fastgen/utils/loading.py:203-260``; only local
+    folders: nothing is fetched)."""
+
+    def __init__(self, model: str | Path) -> None:
+        self.model_dir = Path(model)
+        if not (self.model_dir / "config.json").is_file():
+            raise FileNotFoundError(f"{self.model_dir}: no config.json (a model folder is needed; hub ids are not fetched)")
+
+    def load_model_args(self):
+        """The typed configuration of the folder's architecture."""
+        import json
+
+        from .config import get_architecture
+
+        with open(self.model_dir / "config.json") as f:
+            config = json.load(f)
+        return get_architecture(config).parse(config)
+
+    def load_tokenizer(self):
+        """The folder's tokenizer, or None if it has none."""
+        from .tools.tokenizer import FolderTokenizer
+
+        return FolderTokenizer.maybe(self.model_dir)
+
+
 class Fastgen:
     def __init__(self, engine: Engine, gen_args: GenArgs, stop_tokens: Sequence[int] = ()) -> None:
         self.engine, self.gen_args, self.stop_tokens = engine, gen_args, tuple(stop_tokens)
 
     @classmethod
-    def build(cls, model_dir: str | Path, gen_args: GenArgs = GenArgs(), device: str = "cuda:0",
-              stop_tokens: Optional[Sequence[int]] = None) -> "Fastgen":
-        """Load the model of ``model_dir`` and size its cache
-        (``fastgen/generate.py:139-173``)."""
+    def build(cls, loader: "HfLoader | str | Path", gen_args: GenArgs = GenArgs(), tp_mesh: Any = None,
+              device: str = "cuda:0", stop_tokens: Optional[Sequence[int]] = None) -> "Fastgen":
+        """Load the model of ``loader`` (an :class:`HfLoader` or the folder
+        itself) and size its cache (``fastgen/generate.py:139-173``).
+        ``tp_mesh`` is the reference's tensor-parallel mesh: this engine runs
+        on one GPU and takes None only."""
+        if tp_mesh is not None:
+            raise RuntimeError("fastgen_amd runs on one GPU: tp_mesh must be None")
+        model_dir = loader.model_dir if isinstance(loader, HfLoader) else loader
         device_ = torch.device(device)
         if device_.type != "cuda":
             raise RuntimeError("fastgen_amd runs on a GPU only")  # generate.py:148
         model = Model.from_folder(model_dir, gen_args.dtype, device_)
+        if stop_tokens is None and isinstance(loader, HfLoader):
+            tokenizer = loader.load_tokenizer()
+            stop_tokens = tokenizer.stop_tokens if tokenizer is not None else None
         if stop_tokens is None:
             eos = getattr(model.args, "extra", {}).get("eos_token_id", [])
             stop_tokens = eos if isinstance(eos, (list, tuple)) else [eos]

@@ -210,8 +210,16 @@ def test_reference_style_interface(tiny_b):
     assert set(out) == {f"t{i}" for i in range(5)}
     for i, p in enumerate(tiny_b["prompts"]):
         assert out[f"t{i}"] == plain_greedy(tiny_b["weights"], TINY_B, p, 5 if i == 0 else 8)
-    # sizing from a memory budget (fastgen/utils/tune.py:68-84)
-    fg2 = Fastgen.build(tiny_b["folder"], GenArgs(gpu_gb=0.6, prefill_gb=0.5, dtype=torch.bfloat16))
+    # sizing from a memory budget (fastgen/utils/tune.py:68-84); the reference's way of calling:
+    # a loader object and keywords (fastgen/tools/chat.py:50-65)
+    from fastgen_amd.generate import HfLoader
+
+    loader = HfLoader(tiny_b["folder"])
+    assert loader.load_model_args().n_layers == 3 and loader.load_tokenizer() is None
+    with pytest.raises(RuntimeError, match="one GPU"):
+        Fastgen.build(loader=loader, gen_args=GenArgs(), tp_mesh=object(), device="cuda:0")
+    fg2 = Fastgen.build(loader=loader, gen_args=GenArgs(gpu_gb=0.6, prefill_gb=0.5, dtype=torch.bfloat16),
+                        tp_mesh=None, device="cuda:0")
     per_token = 2 * 3 * 32 * 2 * 3
     pool = fg2.engine.runner.cache.n_pages[0] * 64
     assert pool == pytest.approx((0.1e9 - fg2.engine.model.weight_bytes()) / per_token, abs=64)
