@@ -28,8 +28,9 @@ logger = logging.getLogger(__name__)
 @dataclass
 class GenArgs:
     """Generation options (``fastgen/generate.py:30-59``).  Options of the
-    reference that belong to parts this engine does not have (host cache,
-    CUDA graphs count, fp8, hold-back thresholds) are absent."""
+    reference that belong to parts this engine does not have (fp8 clipping,
+    the hold-back thresholds ``min_prefill`` / ``min_prefill_batch``, which
+    with the reference's defaults never hold anything back) are absent."""
 
     use_sampling: bool = True  # else greedy for every request
     temperature: float = 0.7
@@ -38,7 +39,9 @@ class GenArgs:
     max_batch: int = 256  # most concurrent requests
     max_seq: int = -1  # cache size in tokens, also the cap of one request; negative: from gpu_gb
     max_gen: Optional[int] = None  # default cap of generated tokens
+    host_cache_gb: float = 0  # the reference's host-memory prefix cache: not built, must stay 0
     cache_block: int = 64  # tokens per cache page (the reference's default is 256)
+    num_cuda_graphs: int = 64  # most captured decode steps (the reference: 16); 0: every step runs eagerly
     max_prefill: int = 8192  # token budget of one step
     prefill_gb: float = 0.5  # activation budget, used when sizing the cache
     gpu_gb: float = 20  # memory budget, used when max_seq is negative
@@ -112,6 +115,8 @@ class Fastgen:
         on one GPU and takes None only."""
         if tp_mesh is not None:
             raise RuntimeError("fastgen_amd runs on one GPU: tp_mesh must be None")
+        if gen_args.host_cache_gb:
+            raise RuntimeError("fastgen_amd has no host-memory prefix cache: host_cache_gb must be 0")
         model_dir = loader.model_dir if isinstance(loader, HfLoader) else loader
         device_ = torch.device(device)
         if device_.type != "cuda":
@@ -133,6 +138,7 @@ class Fastgen:
         engine = Engine(model, page_size=gen_args.cache_block, max_tokens=max_seq, max_batch=max_batch,
                         max_step_tokens=gen_args.max_prefill, max_seq=max_seq, seed=gen_args.seed,
                         sync_freq=gen_args.sync_freq)
+        engine.runner.max_graphs = max(0, gen_args.num_cuda_graphs)
         return cls(engine, gen_args, stop_tokens)
 
     def _params(self, pkt: Packet) -> SamplingParams:
