@@ -138,13 +138,14 @@ def test_float32_does_not_depend_on_the_cut(case):
         assert torch.equal(a[rid], b[rid]), rid
 
 
-def test_a_stale_or_foreign_page_is_never_read(case):
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_stale_or_foreign_page_is_never_read(case, dtype):
     """Pages are poisoned with NaN before every step except where the live
     requests hold tokens: what lies beyond a request's length, in free pages
     or in other requests' pages, must not reach its logits."""
     from fastgen_amd.engine import StepEntry
 
-    runner = make_runner(case["folder"], torch.float32, case["page"], 512)
+    runner = make_runner(case["folder"], dtype, case["page"], 512)
     for t in runner.storage.k + runner.storage.v:
         t.fill_(float("nan"))
     toks = case["tokens"]
@@ -152,10 +153,12 @@ def test_a_stale_or_foreign_page_is_never_read(case):
     n = case["lengths"][rid]
     cut = n // 2
     got = [runner.step([StepEntry(rid, toks[rid][:cut], list(range(cut)))])]
-    got.append(runner.step([StepEntry(rid, toks[rid][cut:], list(range(n - cut)))]))
+    got.append(runner.step([StepEntry(rid, toks[rid][cut : n - 3], list(range(n - 3 - cut)))]))
+    for p in range(n - 3, n):  # and the last tokens one by one (the decode kernels)
+        got.append(runner.step([StepEntry(rid, [toks[rid][p]], [0])]).clone())
     got = torch.cat(got).cpu()
     assert torch.isfinite(got).all()
-    assert_close({rid: got}, {rid: case["want"][rid]}, torch.float32, None, "poison")
+    assert_close({rid: got}, {rid: case["want"][rid]}, dtype, case["noise"] if dtype == torch.bfloat16 else None, "poison")
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
