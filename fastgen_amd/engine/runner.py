@@ -153,7 +153,9 @@ class ModelRunner:
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """fp32 logits ``[n_wanted, vocab]`` in the order of the entries and
-        of their ``want`` lists; None if nothing is wanted."""
+        of their ``want`` lists; None if nothing is wanted.  The tensor may be
+        the buffer of a captured step: it holds these logits until the next
+        step; copy what is to be kept."""
         if self.use_graphs and self._is_plain_decode(entries):
             logits = self._graph_step(entries)
         else:
