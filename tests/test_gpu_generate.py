@@ -29,7 +29,7 @@ def tiny_b(tmp_path_factory):
 
 
 def test_greedy_generation_matches_the_plain_implementation(tiny_b):
-    """BASELINE's second workload: prompts of 1, 12, 40, 90 and 150 tokens, 16
+    """Prompts of 1, 12, 40, 90 and 150 tokens, 16
     new tokens each, portions of at most 24 tokens a step beside decodes."""
     from fastgen_amd.engine import Engine
     from fastgen_amd.sampling import SamplingParams
