@@ -77,7 +77,7 @@ class Engine:
         that ended with it."""
         n_run = self.scheduler.plan_decode_run(self.sync_freq) if self.runner.can_graph(len(self.scheduler.running)) else 0
         if n_run:
-            return self._decode_run(n_run)
+            return self._ended(self._decode_run(n_run))
         plan = self.scheduler.plan()
         done: List[Request] = []
         if plan:
@@ -100,7 +100,11 @@ class Engine:
                 sampled = tok.tolist()
             done = self.scheduler.commit(plan, sampled, lps)
             self.n_steps += 1
-        # requests the scheduler ended while planning (alone and out of pages)
+        return self._ended(done)
+
+    def _ended(self, done: List[Request]) -> List[Request]:
+        """``done`` and what else the scheduler ended since the last step (a request alone and out
+        of pages ends while planning); every ended request is reported once."""
         for r in self.scheduler.finished:
             if r not in done:
                 done.append(r)

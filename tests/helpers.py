@@ -80,3 +80,21 @@ def assert_close(got: Mapping[str, torch.Tensor], want: Mapping[str, torch.Tenso
             f"{what} request {rid}: first position over tolerance is "
             f"{int((err > tol).nonzero()[0])} of {len(err)}, worst {worst}: {float(err.max()):.3e} > {tol:.3e}"
         )
+
+
+def write_tiny_tokenizer(folder: Path, n_words: int = 40) -> List[str]:
+    """A word-level tokenizer (``tokenizer.json``, ``tokenizer_config.json`` with
+    an end token and a chat template) in ``folder``; returns its words."""
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import WhitespaceSplit
+
+    words = ["<unk>", "<end>", "<user>", "<bot>"] + [f"w{i}" for i in range(n_words)]
+    tok = Tokenizer(WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = WhitespaceSplit()
+    tok.save(str(folder / "tokenizer.json"))
+    template = "{% for m in messages %}{{ '<user> ' if m['role'] == 'user' else '<bot> ' }}{{ m['content'] }} <end> {% endfor %}<bot>"
+    with open(folder / "tokenizer_config.json", "w") as f:
+        json.dump({"eos_token": {"content": "<end>"}, "chat_template": template}, f)
+    return words
+

@@ -200,3 +200,22 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode == 2
     assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
 
+
+def test_folder_tokenizer(tmp_path):
+    """tokenizer.json and the chat template of tokenizer_config.json
+    (fastgen/utils/tokenizer.py:48-118)."""
+    from helpers import write_tiny_tokenizer
+
+    from fastgen_amd.tools.tokenizer import FolderTokenizer
+
+    assert FolderTokenizer.maybe(tmp_path) is None
+    words = write_tiny_tokenizer(tmp_path)
+    tok = FolderTokenizer.maybe(tmp_path)
+    assert tok.stop_tokens == [words.index("<end>")]
+    ids = tok.encode("w3 w0 w39")
+    assert ids == [words.index(w) for w in ("w3", "w0", "w39")]
+    assert tok.decode(ids) == "w3 w0 w39"
+    dialog = [{"role": "user", "content": "w1 w2"}, {"role": "assistant", "content": "w5"}, {"role": "user", "content": "w7"}]
+    want = "<user> w1 w2 <end> <bot> w5 <end> <user> w7 <end> <bot>".split()
+    assert tok.encode_dialog(dialog) == [words.index(w) for w in want]
+

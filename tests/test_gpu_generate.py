@@ -210,6 +210,14 @@ def test_reference_style_interface(tiny_b):
     assert set(out) == {f"t{i}" for i in range(5)}
     for i, p in enumerate(tiny_b["prompts"]):
         assert out[f"t{i}"] == plain_greedy(tiny_b["weights"], TINY_B, p, 5 if i == 0 else 8)
+    # one generator serves request after request, as the chat tool uses it (fastgen/tools/chat.py:67-80):
+    # every finished request comes out once
+    q2: "queue.Queue" = queue.Queue()
+    gen = fg.generate(q2)
+    for turn in range(3):
+        q2.put(Packet(thread_id=turn, tokens=tiny_b["prompts"][2]))
+        pkt = next(gen)
+        assert pkt.thread_id == turn and pkt.tokens == out["t2"]
     # sizing from a memory budget (fastgen/utils/tune.py:68-84); the reference's way of calling:
     # a loader object and keywords (fastgen/tools/chat.py:50-65)
     from fastgen_amd.generate import HfLoader
@@ -236,6 +244,38 @@ def test_command_line(tiny_b):
     got = [int(x) for x in proc.stdout.strip().splitlines()[0].split(",")]
     assert got == plain_greedy(tiny_b["weights"], TINY_B, prompt, 6)
     assert "tok/s" in proc.stderr
+
+
+def test_command_line_with_a_tokenizer(tiny_b, tmp_path):
+    """A text prompt through the folder's tokenizer and chat template; and the
+    dialogue loop on standard input (a turn, /r, a turn, /q)."""
+    import shutil
+
+    from helpers import write_tiny_tokenizer
+
+    from fastgen_amd.tools.tokenizer import FolderTokenizer
+
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(tiny_b["folder"], folder)
+    write_tiny_tokenizer(folder, n_words=380)  # as many words as the model has tokens
+    tok = FolderTokenizer(folder)
+    base = [sys.executable, str(REPO / "bin" / "fgchat"), str(folder), "--max-tokens", "5", "--temperature", "0",
+            "--dtype", "float32", "--max-seq", "256", "--gpu-gb", "1"]
+    proc = subprocess.run(base + ["--prompt", "w1 w2 w3"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    ids = tok.encode_dialog([{"role": "user", "content": "w1 w2 w3"}])
+    want = plain_greedy(tiny_b["weights"], TINY_B, ids, 5)
+    stop = tok.stop_tokens[0]
+    if stop in want:  # generation ends with the stop token
+        want = want[: want.index(stop) + 1]
+    lines = proc.stdout.strip().splitlines()
+    assert [int(x) for x in lines[0].split(",")] == want
+    assert lines[1] == tok.decode([t for t in want if t != stop])
+    # the dialogue loop: the first answer is the same generation
+    proc = subprocess.run(base, input="w1 w2 w3\n/r\nw1 w2 w3\n/q\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    answers = [l.replace("> ", "") for l in proc.stdout.splitlines() if l.replace("> ", "").strip()]
+    assert len(answers) == 2 and answers[0] == answers[1] == lines[1]
 
 
 def test_smoke_entry():
