@@ -72,6 +72,11 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    def abort(self, rid: Hashable) -> bool:
+        """End a request before it is done; it comes out of the next ``step`` with ``finish_reason``
+        ``aborted`` and what it has generated so far."""
+        return self.scheduler.abort(rid)
+
     def step(self) -> List[Request]:
         """One step of the model over what the scheduler picks; the requests
         that ended with it."""
@@ -136,7 +141,15 @@ class Engine:
                  ) -> List[List[int]]:
         """Generated ids for every prompt, in the order of the prompts."""
         plist = list(params) if isinstance(params, (list, tuple)) else [params] * len(prompts)
-        rids = [self.add_request(p, sp) for p, sp in zip(prompts, plist)]
+        rids: List[Hashable] = []
+        try:
+            for p, sp in zip(prompts, plist):
+                rids.append(self.add_request(p, sp))
+        except Exception:
+            for rid in rids:  # all or nothing: a refused prompt leaves none of the call's requests behind
+                self.abort(rid)
+            self.scheduler.finished.clear()
+            raise
         out: Dict[Hashable, List[int]] = {}
         while self.has_work():
             for r in self.step():
@@ -192,6 +205,6 @@ class Engine:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         for r in list(self.scheduler.running):  # the measurement is over: let go of the batch
-            self.scheduler._finish(r, "aborted")
+            self.abort(r.rid)
         self.scheduler.finished.clear()
         return dt

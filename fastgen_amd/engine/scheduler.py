@@ -107,6 +107,17 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def abort(self, rid) -> bool:
+        """End the request ``rid`` now, waiting or running: its pages and slot go back and it is
+        reported as ended with reason ``aborted``.  False if there is no such request."""
+        for req in list(self.running) + list(self.waiting):
+            if req.rid == rid:
+                if req in self.waiting:
+                    self.waiting.remove(req)
+                self._finish(req, "aborted")
+                return True
+        return False
+
     # --------------------------------------------------------------- plan
     def _preempt(self, victim: Request) -> None:
         self.cache.release(victim.rid)

@@ -201,6 +201,26 @@ def test_max_batch_and_first_come_first_served():
     assert first_seen[2] == 3  # as soon as request 0 (3 new tokens) has ended
 
 
+def test_abort_gives_pages_and_slot_back():
+    """A running request and a waiting one are ended from outside: pages and
+    slot return, the others go on undisturbed."""
+    s = mk(cache_pages=16, max_batch=2, budget=64)
+    reqs = [Request(i, list(range(20)), max_new=6) for i in range(3)]
+    for r in reqs:
+        s.add(r)
+    plan = s.plan()  # requests 0 and 1 run, 2 waits
+    for e in plan:
+        s.cache.advance(e.request.rid, e.n)
+    s.commit(plan, [fake_token(e.request, e.start + e.n) for e in plan if e.wants_logits])
+    assert s.abort(0) and s.abort(2) and not s.abort(99)
+    assert [r.finish_reason for r in reqs] == ["aborted", None, "aborted"]
+    assert [r.rid for r in s.finished] == [0, 2] and s.cache.live_requests() == [1]
+    s.cache.check()
+    drive(s)
+    assert reqs[1].finish_reason == "length" and len(reqs[1].generated) == 6
+    assert s.cache.live_requests() == [] and s.cache.free_pages() == 16 and s.cache.free_slots() == 2
+
+
 def test_stop_ids_and_caps():
     s = mk(max_seq=20)
     r = Request("a", [1, 2, 3], max_new=50)
