@@ -82,6 +82,41 @@ def test_decode_batches_between_the_captured_sizes(tiny_b, dtype):
     eng.runner.cache.check()
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_serving_load_matches_the_plain_implementation(seed, tmp_path):
+    """Requests of random lengths, caps and stop tokens through a small pool
+    (so that some are preempted and recomputed) with few slots, prompt portions
+    beside decodes, decode runs between host checks: every request's tokens are
+    those the plain implementation generates for it alone."""
+    import random
+
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    rng = random.Random(seed)
+    w = plain_random_weights(TINY_A, 5)
+    w = {k: v * 8 if ("q_proj" in k or "k_proj" in k or "embed" in k) else v for k, v in w.items()}
+    folder = save_model_folder(tmp_path / "load", TINY_A, w)
+    g = torch.Generator().manual_seed(seed)
+    reqs = []
+    for _ in range(22):
+        prompt = torch.randint(0, 256, (rng.randint(1, 60),), generator=g).tolist()
+        max_new = rng.randint(1, 24)
+        alone = plain_greedy(w, TINY_A, prompt, max_new)
+        stop = ()
+        if rng.random() < 0.4 and len(alone) > 2:
+            stop = (alone[rng.randrange(1, len(alone))],)  # a token it will generate: ends there
+            alone = alone[: alone.index(stop[0]) + 1]
+        reqs.append((prompt, SamplingParams(temperature=0.0, max_new_tokens=max_new, stop_ids=stop), alone))
+    eng = Engine.from_folder(folder, torch.float32, page_size=16, max_tokens=176, max_batch=5, max_step_tokens=32,
+                             sync_freq=4)
+    got = eng.generate([r[0] for r in reqs], [r[1] for r in reqs])
+    assert got == [r[2] for r in reqs]
+    assert eng.scheduler.n_preemptions > 0
+    assert eng.runner.cache.live_requests() == []
+    eng.runner.cache.check()
+
+
 def test_preemption_gives_the_same_tokens(tiny_b):
     from fastgen_amd.engine import Engine
     from fastgen_amd.sampling import SamplingParams
