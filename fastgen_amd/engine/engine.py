@@ -32,6 +32,8 @@ class Engine:
         elif cap:
             max_seq = min(max_seq, cap)
         self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit)
+        # no request gets longer than the scheduler lets it: block tables need not be wider
+        self.runner.table_width = min(self.runner.table_width, -(-self.scheduler.max_seq // page_size))
         self.sampler = Sampler(model.device)
         self.seed = seed
         # decode steps between host checks for finished requests when nothing waits for admission

@@ -33,20 +33,34 @@ def graph_capacity_for(n: int) -> int:
     return -(-n // step) * step
 
 
-class _DecodeGraph:
-    """One captured decode step for a fixed number of sequences.
+def graph_table_width_for(n_pages: int, limit: int) -> int:
+    """The block-table width of the captured step that serves requests holding
+    up to ``n_pages`` pages: powers of two from 16 on, at most ``limit`` (the
+    widest a request can get).  The step's vectors are copied to the device at
+    every replay: tables as wide as the cache would make that copy as large as
+    the cache's page count times the batch."""
+    w = 16
+    while w < n_pages:
+        w *= 2
+    return max(1, min(w, limit))
 
-    The step's int32 vectors live in a device buffer of fixed layout (block
-    tables as wide as a request can get); a replay copies the new values in
-    and runs the captured kernels, which read lengths and pages from that
-    buffer.  A smaller batch is filled up with stand-in sequences that write
-    nothing; a graph is captured when a batch of its capacity first occurs.
+
+class _DecodeGraph:
+    """One captured decode step for a fixed number of sequences and a fixed
+    width of their block tables.
+
+    The step's int32 vectors live in a device buffer of fixed layout; a replay
+    copies the new values in and runs the captured kernels, which read lengths
+    and pages from that buffer.  A smaller batch is filled up with stand-in
+    sequences that write nothing; a graph is captured when a batch of its
+    capacity and table width first occurs.
     """
 
-    def __init__(self, runner: "ModelRunner", entries: Sequence[StepEntry]) -> None:
+    def __init__(self, runner: "ModelRunner", entries: Sequence[StepEntry], table_width: int) -> None:
         model, cache = runner.model, runner.cache
         self.capacity = graph_capacity_for(len(entries))
-        packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, runner.table_width, self.capacity)
+        self.table_width = table_width
+        packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, table_width, self.capacity)
         self.layout = (tuple(int(o) for o in offs), tuple(shapes))
         # a ring of pinned staging buffers: the host may run several steps ahead of the device
         self.staging = [torch.empty(packed.size, dtype=torch.int32, pin_memory=True) for _ in range(runner.run_ahead)]
@@ -55,7 +69,7 @@ class _DecodeGraph:
         self.staging[0].numpy()[:] = packed
         self.packed = self.staging[0].to(model.device)
         self.ctx = context_from_packed(self.packed, offs, shapes, host, cache.page_size, model.dtype)
-        self.ctx.graph_capacity = runner.table_width * cache.page_size
+        self.ctx.graph_capacity = table_width * cache.page_size  # the longest sequence this step may meet
         # warm up outside the capture (libraries load, the matrix library picks its kernels), then capture
         side = torch.cuda.Stream(device=model.device)
         side.wait_stream(torch.cuda.current_stream(model.device))
@@ -78,7 +92,7 @@ class _DecodeGraph:
         ``entries``: the step before sampled them and the host has not seen them."""
         n = len(entries)
         packed, offs, shapes, host = pack_context(entries, runner.cache, None if tokens_on_device is not None
-                                                  else runner.model.vocab_size, runner.table_width, self.capacity)
+                                                  else runner.model.vocab_size, self.table_width, self.capacity)
         if (tuple(int(o) for o in offs), tuple(shapes)) != self.layout:
             raise RuntimeError("decode graph: the step's layout differs from the captured one")
         i = self.turn = (self.turn + 1) % len(self.staging)
@@ -120,7 +134,7 @@ class ModelRunner:
         self.use_graphs = (os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and not model.state_needs()
                            and model.capturable())
         self.table_width = max(1, max(pages, default=1))
-        self.graphs: Dict[int, _DecodeGraph] = {}
+        self.graphs: Dict[Tuple[int, int], _DecodeGraph] = {}  # (capacity, table width) -> step, oldest use first
         self.graph_pool = None
         self.max_graphs = 64
         self.run_ahead = 16  # steps the host may prepare before the device has run them
@@ -174,14 +188,20 @@ class ModelRunner:
         ) and self.can_graph(len(entries))
 
     def can_graph(self, n: int) -> bool:
-        """Whether a decode batch of ``n`` has, or may still get, a captured step."""
-        return self.use_graphs and (graph_capacity_for(n) in self.graphs or len(self.graphs) < self.max_graphs)
+        """Whether decode batches run from captured steps."""
+        return self.use_graphs and self.max_graphs > 0
 
     def _graph_for(self, entries: Sequence[StepEntry]) -> _DecodeGraph:
-        cap = graph_capacity_for(len(entries))
-        g = self.graphs.get(cap)
+        """The captured step for these entries (whose pages are reserved): by batch capacity and
+        block-table width.  At most ``max_graphs`` are kept; the one unused longest gives way."""
+        held = max(self.cache.n_table_entries(e.rid, g) for e in entries for g in range(self.cache.n_groups))
+        key = (graph_capacity_for(len(entries)), graph_table_width_for(held, self.table_width))
+        g = self.graphs.pop(key, None)
         if g is None:
-            g = self.graphs[cap] = _DecodeGraph(self, entries)
+            while len(self.graphs) >= self.max_graphs:
+                self.graphs.pop(next(iter(self.graphs)))
+            g = _DecodeGraph(self, entries, key[1])
+        self.graphs[key] = g  # most recently used last
         return g
 
     def decode_run(self, entries: Sequence[StepEntry], n_steps: int, sample) -> torch.Tensor:

@@ -60,8 +60,9 @@ def test_decode_batches_between_the_captured_sizes(tiny_b, dtype):
     eng = Engine.from_folder(tiny_b["folder"], dtype, page_size=16, max_tokens=21 * 96, max_batch=32,
                              max_step_tokens=256)
     got = eng.generate(prompts, params)
-    caps = sorted(eng.runner.graphs)
+    caps = sorted({cap for cap, _ in eng.runner.graphs})  # keys: (sequences, block-table width)
     assert caps and max(caps) == 24 and 17 not in caps and 21 not in caps  # padded, not captured per size
+    assert {w for _, w in eng.runner.graphs} == {16}  # short requests: narrow tables, not the pool's 126 pages
     if dtype == torch.float32:
         want = [plain_greedy(tiny_b["weights"], TINY_B, p, sp.max_new_tokens) for p, sp in zip(prompts, params)]
         assert got == want
