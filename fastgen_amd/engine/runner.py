@@ -199,6 +199,7 @@ class ModelRunner:
         g = self.graphs.pop(key, None)
         if g is None:
             while len(self.graphs) >= self.max_graphs:
+                torch.cuda.synchronize(self.model.device)  # its last replay may still be running
                 self.graphs.pop(next(iter(self.graphs)))
             g = _DecodeGraph(self, entries, key[1])
         self.graphs[key] = g  # most recently used last

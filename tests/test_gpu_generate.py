@@ -118,6 +118,23 @@ def test_random_serving_load_matches_the_plain_implementation(seed, tmp_path):
     eng.runner.cache.check()
 
 
+def test_captured_steps_give_way_to_new_ones(tiny_b):
+    """With room for two captured steps, batches of four sizes still decode
+    from captured steps (the least recently used one gives way) and give the
+    tokens of the plain implementation."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=1024, max_batch=4,
+                             max_step_tokens=64, sync_freq=3)
+    eng.runner.max_graphs = 2
+    prompts = tiny_b["prompts"][:4]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=n) for n in (5, 9, 13, 17)]  # batch shrinks 4, 3, 2, 1
+    got = eng.generate(prompts, params)
+    assert got == [plain_greedy(tiny_b["weights"], TINY_B, p, sp.max_new_tokens) for p, sp in zip(prompts, params)]
+    assert len(eng.runner.graphs) == 2 and {cap for cap, _ in eng.runner.graphs} == {1, 2}
+
+
 def test_preemption_gives_the_same_tokens(tiny_b):
     from fastgen_amd.engine import Engine
     from fastgen_amd.sampling import SamplingParams
