@@ -31,7 +31,6 @@ LLAMA_8B = dict(
                       original_max_position_embeddings=8192),
     tie_word_embeddings=False, max_position_embeddings=131072,
 )
-FULL_LAYERS = 32
 PROMPT_LEN = 2048
 CONTEXT_LEN = 8192  # capacity per request
 PAGE = 64
@@ -44,6 +43,16 @@ LLAMA_3B = dict(
                       original_max_position_embeddings=8192),
     tie_word_embeddings=True, max_position_embeddings=131072,
 )
+
+
+LLAMA_70B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=8192, intermediate_size=28672, num_hidden_layers=80,
+    num_attention_heads=64, num_key_value_heads=8, rms_norm_eps=1e-5, vocab_size=128256, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=False, max_position_embeddings=131072,
+)
+SHAPES = {"8b": ("llama-3.1-8b-shape-random", LLAMA_8B), "70b": ("llama-3.1-70b-shape-random", LLAMA_70B)}
 
 
 def serve_workload(n_requests: int = 256) -> int:
@@ -127,7 +136,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="layer sizes: Llama 3.1 8B (default, the benchmark's configuration) or 70B (141 GB of weights)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--workload", choices=["decode", "serve", "readme"], default="decode",
@@ -147,7 +158,10 @@ def main() -> int:
     from fastgen_amd.engine import Engine
 
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[a.dtype]
-    cfg = dict(LLAMA_8B, num_hidden_layers=a.layers)
+    model_name, shape = SHAPES[a.shape]
+    full_layers = shape["num_hidden_layers"]
+    a.layers = a.layers or full_layers
+    cfg = dict(shape, num_hidden_layers=a.layers)
     batches = sorted({a.batch} | (set() if a.no_points else {1, 64}))
     max_b = max(batches)
     t0 = time.time()
@@ -194,10 +208,10 @@ def main() -> int:
         "ms_per_step": round(r["ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
         "config": {
-            "model": "llama-3.1-8b-shape-random", "global_batch": a.batch, "seq_len": CONTEXT_LEN,
-            "prompt_len": PROMPT_LEN, "parallelism": "none", "layers": L, "layers_full": FULL_LAYERS,
+            "model": model_name, "global_batch": a.batch, "seq_len": CONTEXT_LEN,
+            "prompt_len": PROMPT_LEN, "parallelism": "none", "layers": L, "layers_full": full_layers,
             "hidden": D, "heads": H, "kv_heads": KV, "head_dim": hd, "ffn": F, "vocab": V, "page_size": PAGE,
-            "rope_theta": cfg["rope_theta"], "rope_factor": 8.0, "norm_eps": cfg["rms_norm_eps"],
+            "rope_theta": cfg["rope_theta"], "rope_factor": cfg["rope_scaling"]["factor"], "norm_eps": cfg["rms_norm_eps"],
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
