@@ -636,16 +636,47 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
     if (NPT == 2 && k0 + TILE <= pos_last) stash(s0 + NPT - 1, kreg[NPT - 1], vreg[NPT - 1]);
   };
   if (NSLOT == 2 * NPT) {
-    // pass i is read from its slots while pass i+1 is written to the other slots and the loads of
-    // pass i+2 are in flight: one barrier a pass
-    fetch_pass(k_first);
-    stash_pass(k_first, 0);
-    if (k_first + STEP <= pos_last) fetch_pass(k_first + STEP);
+    // Pass i is read from its slots while pass i+1 arrives in the other slots: one barrier a pass.
+    // A tile that is one whole page inside the key range goes from memory straight into LDS (a
+    // lane's 16 bytes land at the wave's base + 16 * lane: the order the copy through registers
+    // stores them in, too) and costs neither registers nor instructions; the tiles at the edges
+    // of the range go through registers, where they are masked.
+    auto bring = [&](int k0, int slot) {
+      if (k0 > pos_last) return;  // uniform
+      if (PERM && (page_size & 63) == 0 && k0 >= first_min && k0 + TILE - 1 <= pos_last) {
+        const int kin = pager.in_page(k0);
+        const bf16_t* base_k = k_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)kin * HD;
+        const bf16_t* base_v = v_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)(kin >> 3) * 128;
+        const size_t v_block = (size_t)(page_size >> 3) * 128;
+#pragma unroll
+        for (int j = 0; j < KN; ++j) {
+          const int w = threadIdx.x + NT * j;
+          if (w < KTOT)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base_k + (size_t)w * 8),
+                                             (__attribute__((address_space(3))) void*)(k_lds[slot] + (size_t)(w - lane) * 8),
+                                             16, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < VN; ++j) {
+          const int w = threadIdx.x + NT * j;
+          if (w < VTOT)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(base_v + (size_t)(w >> 7) * v_block + (size_t)(w & 127) * 8),
+                (__attribute__((address_space(3))) void*)(v_lds[slot] + (size_t)(w - lane) * 8), 16, 0, 0);
+        }
+      } else {
+        fetch(k0, kreg[0], vreg[0]);
+        stash(slot, kreg[0], vreg[0]);
+      }
+    };
+    bring(k_first, 0);
+    bring(k_first + TILE, 1);
     int s0 = 0;
     for (int k0 = k_first; k0 <= pos_last; k0 += STEP, s0 ^= NPT) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of pass k0 has landed in LDS
       __syncthreads();  // pass k0 is complete in its slots; nobody reads the other slots any more
-      if (k0 + STEP <= pos_last) stash_pass(k0 + STEP, s0 ^ NPT);
-      if (k0 + 2 * STEP <= pos_last) fetch_pass(k0 + 2 * STEP);
+      bring(k0 + STEP, s0 ^ NPT);
+      bring(k0 + STEP + TILE, (s0 ^ NPT) + 1);
       const int mine = k0 + par * TILE;
       if (mine <= pos_last) compute(mine, s0 + par);
     }
