@@ -536,10 +536,10 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
   constexpr int KTOT = TILE * KCH, VTOT = NDB * 8 * 16;  // chunks of a K tile, of a V tile
   constexpr int KN = (KTOT + NT - 1) / NT;     // K chunks a thread copies per tile
   constexpr int VN = (VTOT + NT - 1) / NT;     // V chunks a thread copies per tile
-  bf16x8 kreg[NPT][KN], vreg[NPT][VN];
-  // The next tiles' chunks are fetched into registers while the current ones are computed from
-  // LDS.  Loads are never conditional within a tile: addresses are clamped into the item's key
-  // range, value slots outside it are masked, keys outside it give scores that the select discards.
+  bf16x8 kreg[KN], vreg[VN];
+  // A tile's chunks on their way through registers.  Loads are never conditional within a tile:
+  // addresses are clamped into the item's key range, value slots outside it are masked, keys
+  // outside it give scores that the select discards.
   auto fetch = [&](int k0, bf16x8(&kr)[KN], bf16x8(&vr)[VN]) {
     if (PERM && (page_size & 63) == 0 && k0 >= first_min && k0 + TILE - 1 <= pos_last) {
       // The whole tile lies in one page and inside the key range: K's four 16-key blocks are 64*HD
@@ -627,14 +627,6 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
   };
   const int k_first = (first_min / TILE) * TILE;
   constexpr int STEP = NPT * TILE;  // keys per pass of the loop
-  auto fetch_pass = [&](int k0) {  // uniform conditions: a tile wholly beyond the range is not fetched
-    fetch(k0, kreg[0], vreg[0]);
-    if (NPT == 2 && k0 + TILE <= pos_last) fetch(k0 + TILE, kreg[NPT - 1], vreg[NPT - 1]);
-  };
-  auto stash_pass = [&](int k0, int s0) {
-    stash(s0, kreg[0], vreg[0]);
-    if (NPT == 2 && k0 + TILE <= pos_last) stash(s0 + NPT - 1, kreg[NPT - 1], vreg[NPT - 1]);
-  };
   if (NSLOT == 2 * NPT) {
     // Pass i is read from its slots while pass i+1 arrives in the other slots: one barrier a pass.
     // A tile that is one whole page inside the key range goes from memory straight into LDS (a
@@ -665,8 +657,8 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
                 (__attribute__((address_space(3))) void*)(v_lds[slot] + (size_t)(w - lane) * 8), 16, 0, 0);
         }
       } else {
-        fetch(k0, kreg[0], vreg[0]);
-        stash(slot, kreg[0], vreg[0]);
+        fetch(k0, kreg, vreg);
+        stash(slot, kreg, vreg);
       }
     };
     bring(k_first, 0);
@@ -681,12 +673,13 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
       if (mine <= pos_last) compute(mine, s0 + par);
     }
   } else {
-    fetch_pass(k_first);
+    // one tile at a time: the next tile's chunks fly into registers during this tile's MFMAs
+    fetch(k_first, kreg, vreg);
     for (int k0 = k_first; k0 <= pos_last; k0 += STEP) {
       __syncthreads();  // the previous tile is no longer read
-      stash_pass(k0, 0);
+      stash(0, kreg, vreg);
       __syncthreads();
-      if (k0 + STEP <= pos_last) fetch_pass(k0 + STEP);  // flies during this tile's MFMAs
+      if (k0 + STEP <= pos_last) fetch(k0 + STEP, kreg, vreg);
       compute(k0, 0);
     }
   }
