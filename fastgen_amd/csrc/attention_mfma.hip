@@ -633,12 +633,14 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
     // lane's 16 bytes land at the wave's base + 16 * lane: the order the copy through registers
     // stores them in, too) and costs neither registers nor instructions; the tiles at the edges
     // of the range go through registers, where they are masked.
-    auto bring = [&](int k0, int slot) {
+    // page: the page of key k0, looked up a pass earlier so that nobody waits for the table here
+    auto page_ahead = [&](int k0) { return pager.page_of(min(k0, pos_last)); };
+    auto bring = [&](int k0, int slot, int page) {
       if (k0 > pos_last) return;  // uniform
       if (PERM && (page_size & 63) == 0 && k0 >= first_min && k0 + TILE - 1 <= pos_last) {
         const int kin = pager.in_page(k0);
-        const bf16_t* base_k = k_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)kin * HD;
-        const bf16_t* base_v = v_pages + ((size_t)pager.page_of(k0) * n_kv + kvh) * head_elems + (size_t)(kin >> 3) * 128;
+        const bf16_t* base_k = k_pages + ((size_t)page * n_kv + kvh) * head_elems + (size_t)kin * HD;
+        const bf16_t* base_v = v_pages + ((size_t)page * n_kv + kvh) * head_elems + (size_t)(kin >> 3) * 128;
         const size_t v_block = (size_t)(page_size >> 3) * 128;
 #pragma unroll
         for (int j = 0; j < KN; ++j) {
@@ -661,14 +663,17 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
         stash(slot, kreg, vreg);
       }
     };
-    bring(k_first, 0);
-    bring(k_first + TILE, 1);
+    int page_a = page_ahead(k_first + STEP), page_b = page_ahead(k_first + STEP + TILE);
+    bring(k_first, 0, page_ahead(k_first));
+    bring(k_first + TILE, 1, page_ahead(k_first + TILE));
     int s0 = 0;
     for (int k0 = k_first; k0 <= pos_last; k0 += STEP, s0 ^= NPT) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of pass k0 has landed in LDS
       __syncthreads();  // pass k0 is complete in its slots; nobody reads the other slots any more
-      bring(k0 + STEP, s0 ^ NPT);
-      bring(k0 + STEP + TILE, (s0 ^ NPT) + 1);
+      bring(k0 + STEP, s0 ^ NPT, page_a);
+      bring(k0 + STEP + TILE, (s0 ^ NPT) + 1, page_b);
+      page_a = page_ahead(k0 + 2 * STEP);
+      page_b = page_ahead(k0 + 2 * STEP + TILE);
       const int mine = k0 + par * TILE;
       if (mine <= pos_last) compute(mine, s0 + par);
     }

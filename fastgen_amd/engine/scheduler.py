@@ -138,12 +138,11 @@ class Scheduler:
     def _fits(self, req: Request, n: int) -> int:
         """The largest ``m <= n`` such that ``m`` more tokens of ``req`` fit in
         the pages it holds plus the free ones."""
-        lo = 0
         for g in range(self.cache.n_groups):
             held = self.cache.n_table_entries(req.rid, g)
             room = (held + self.cache.free_pages(g)) * self.cache.page_size - self.cache.length(req.rid)
             n = min(n, room)
-        return max(lo, n)
+        return max(0, n)
 
     def plan(self) -> List[PlannedEntry]:
         entries: List[PlannedEntry] = []
