@@ -15,9 +15,10 @@
 // page layout every operand load of a wave is 1 KB of contiguous memory.
 //
 //  * fg_attn_split (decode and very short portions, <= 16 rows an item): the
-//    key range of an item is cut into splits (grid.x) and a split's tiles are
-//    dealt to the 4 waves, which stream K and V straight from the pages;
-//    partial (max, sum, O) go to scratch and fg_attn_combine merges them.
+//    key ranges of the items are cut into chunks of equal size (fg_attn_plan,
+//    on the device), a chunk is a workgroup whose tiles are dealt to its 4
+//    waves, which stream K and V straight from the pages; the chunks' partial
+//    (max, sum, O) go to scratch and a combine kernel merges them.
 //  * fg_attn_tile (prompt portions, up to 128 rows an item): K and V tiles are
 //    staged in LDS and shared by the workgroup's waves.
 //
@@ -201,23 +202,124 @@ __device__ __forceinline__ void load_q(bf16x8 (&qop)[NKS], const bf16_t* qrow, b
 }
 
 // ------------------------------------------------------------------ split
-// grid (n_splits, n_kv, n_items), 256 threads.  items: [n_items][4] = sequence,
-// flat index of the first token, number of tokens, position of the first
-// token; n_tok * (H / KV) <= 16.
+// The key ranges of the items are cut into chunks of the same number of tiles for every item, so that
+// a long sequence gives many workgroups and a short one few, each with about the same work; a plan
+// kernel does the cutting on the device from the items alone, so that a captured step cuts anew
+// for the lengths of every replay.
+//
+// plan: int32 [4 + 8 * max_chunks]
+//   [0] tiles per chunk, [1] chunks in use;
+//   from [4] on, 8 ints a chunk, the chunks of an item one after the other: the item's record
+//   (sequence, first flat token, tokens, first position), first tile, end tile, chunks of the item
+//   (0: this chunk is not in use), number of this chunk among its item's.
+#define COMBINE_MAX_SPLITS 256
+#define COMBINE_ROWS_MAX_GROUPS 8192  // up to this many workgroups the combine takes a workgroup a row
+constexpr int PLAN_HEAD = 4;
+
+// tiles an item's rows see: [t_lo, t_hi]
+__device__ __forceinline__ void item_tiles(const Item& it, int window, int& t_lo, int& t_hi) {
+  const int pos_last = it.pos0 + it.n_tok - 1;
+  const int first_min = window > 0 && it.pos0 - window + 1 > 0 ? it.pos0 - window + 1 : 0;
+  t_lo = first_min / TILE;
+  t_hi = pos_last / TILE;
+}
+
+// One workgroup.  Tiles per chunk: the smallest multiple of min_tiles (at least min_tiles) with which
+// all chunks fit into max_chunks (> n_items) and no item has more than COMBINE_MAX_SPLITS.
+__global__ __launch_bounds__(256) void attn_plan_kernel(const int* __restrict__ items, int n_items, int window,
+                                                        int max_chunks, int min_tiles, int* __restrict__ plan) {
+  __shared__ int red_s[256], red_m[256];
+  __shared__ int carry;
+  const int tid = threadIdx.x;
+  int tot = 0, mx = 0;
+  for (int i = tid; i < n_items; i += 256) {
+    int lo, hi;
+    item_tiles(load_item(items, i), window, lo, hi);
+    tot += hi - lo + 1;
+    mx = max(mx, hi - lo + 1);
+  }
+  red_s[tid] = tot;
+  red_m[tid] = mx;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (tid < w) {
+      red_s[tid] += red_s[tid + w];
+      red_m[tid] = max(red_m[tid], red_m[tid + w]);
+    }
+    __syncthreads();
+  }
+  tot = red_s[0];
+  mx = red_m[0];
+  __syncthreads();
+  // sum over items of ceil(tiles / ts) <= tot / ts + n_items <= max_chunks
+  const int room = max_chunks - n_items;
+  int ts = max((tot + room - 1) / room, (mx + COMBINE_MAX_SPLITS - 1) / COMBINE_MAX_SPLITS);
+  ts = max(1, (ts + min_tiles - 1) / min_tiles) * min_tiles;
+  int* chunks = plan + PLAN_HEAD;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int i0 = 0; i0 < n_items; i0 += 256) {
+    const int i = i0 + tid;
+    Item it{0, 0, 0, 0};
+    int lo = 0, hi = -1, c = 0;
+    if (i < n_items) {
+      it = load_item(items, i);
+      item_tiles(it, window, lo, hi);
+      c = (hi - lo + ts) / ts;
+    }
+    // inclusive scan of c over the workgroup
+    red_s[tid] = c;
+    __syncthreads();
+    for (int w = 1; w < 256; w <<= 1) {
+      const int add = tid >= w ? red_s[tid - w] : 0;
+      __syncthreads();
+      red_s[tid] += add;
+      __syncthreads();
+    }
+    const int first = carry + red_s[tid] - c;
+    for (int sp = 0; sp < c; ++sp) {
+      int* rec = chunks + (size_t)(first + sp) * 8;
+      *(int4*)rec = int4{it.seq, it.tok0, it.n_tok, it.pos0};
+      *(int4*)(rec + 4) = int4{lo + sp * ts, min(hi + 1, lo + (sp + 1) * ts), c, sp};
+    }
+    __syncthreads();
+    if (tid == 255) carry += red_s[255];
+    __syncthreads();
+  }
+  const int used = carry;
+  for (int j = used + tid; j < max_chunks; j += 256) {
+    int* rec = chunks + (size_t)j * 8;
+    *(int4*)rec = int4{0, 0, 0, 0};
+    *(int4*)(rec + 4) = int4{0, 0, 0, 0};
+  }
+  if (tid == 0) {
+    plan[0] = ts;
+    plan[1] = used;
+  }
+}
+
+// grid (n_kv, max_chunks), 256 threads: one chunk of one item (a run of at most 16 rows:
+// n_tok * (H / KV) <= 16) for one kv head.  An item of one chunk writes its output rows; of more, the
+// chunk's (max, sum, O) go to part_o / part_ml at row (chunk * n_kv + kv head) * 16 + row.
 template <bool PERM /* the page's value slots are permuted: page_size % 32 == 0 */>
 __global__ __launch_bounds__(256) void attn_split_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items,
+    const int* __restrict__ block_table, int bt_stride, const int* __restrict__ plan,
     float* __restrict__ part_o, float* __restrict__ part_ml, int n_heads, int n_kv, int page_size,
     int page_shift, float scale, int window) {
   __shared__ float o_s[2][16][HD + 1];
   __shared__ float ml_s[2][16][2];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
-  const int split = blockIdx.x, n_splits = gridDim.x, kvh = blockIdx.y, item = blockIdx.z;
+  const int kvh = blockIdx.x, chunk = blockIdx.y;
   const int G = n_heads / n_kv;
-  const Item it = load_item(items, item);
+  const int* rec = plan + PLAN_HEAD + (size_t)chunk * 8;
+  const int4 rec_a = *(const int4*)rec, rec_b = *(const int4*)(rec + 4);
+  if (rec_b.z == 0) return;  // uniform: a chunk that is not in use
+  const Item it{rec_a.x, rec_a.y, rec_a.z, rec_a.w};
+  const int t_begin = rec_b.x, t_end = rec_b.y;
+  const bool alone = rec_b.z == 1;  // the item's only chunk
   const Pager pager{block_table + (size_t)it.seq * bt_stride, page_size, page_shift};
   const KvLayout lay(page_size, HD);
 
@@ -232,11 +334,6 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   }
   bf16x8 qop[1][NKS];
   load_q(qop[0], q + (size_t)(it.tok0 + my_tok) * q_stride + (size_t)(kvh * G + my_head) * HD, my_row);
-
-  const int t_lo = first_min / TILE, t_hi = pos_last / TILE;
-  const int per_split = (t_hi - t_lo + 1 + n_splits - 1) / n_splits;
-  const int t_begin = t_lo + split * per_split;
-  const int t_end = min(t_hi + 1, t_begin + per_split);
 
   float m_[1] = {-INFINITY}, l_[1] = {0.f};
   f32x4 o_[1][NDB];
@@ -336,7 +433,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   take(0);
   if (r16 >= it.n_tok * G) return;
   const int t_out = it.tok0 + r16 / G, h_out = kvh * G + r16 % G;
-  if (n_splits == 1) {
+  if (alone) {
     bf16_t* orow = out + (size_t)t_out * out_stride + (size_t)h_out * HD;
     const float inv = 1.f / l;
 #pragma unroll
@@ -347,7 +444,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
       *(bf16x4*)(orow + 16 * db + 4 * g) = v;
     }
   } else {
-    const size_t row = (((size_t)item * n_kv + kvh) * n_splits + split) * 16 + r16;
+    const size_t row = ((size_t)chunk * n_kv + kvh) * 16 + r16;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) *(f32x4*)(part_o + row * HD + 16 * db + 4 * g) = o[db];
     if (g == 0) {
@@ -357,36 +454,42 @@ __global__ __launch_bounds__(256) void attn_split_kernel(
   }
 }
 
-// grid (16 rows, n_kv, n_items), one thread per head dimension (at least one wave).  The splits'
-// maxima and sums are read by the first wave, one split a lane, and the partial outputs eight at a
-// time: the kernel is a chain of dependent reads, so what it costs is how long that chain is.
-#define COMBINE_MAX_SPLITS 256
-__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                    const int* __restrict__ items, bf16_t* __restrict__ out, int out_stride,
-                                    int n_heads, int n_kv, int n_splits) {
-  __shared__ float f_s[COMBINE_MAX_SPLITS];  // weight of each split's partial output: 2^(m_s - M) / L
-  const int r = blockIdx.x, kvh = blockIdx.y, item = blockIdx.z, d = threadIdx.x;
+// Two kernels add up the chunks of the items that have several, in chunk order: the workgroups of an
+// item's first chunk do it, all others leave as soon as they have their chunk's record (a wave that
+// has asked for more has to wait for it before it can end, and most workgroups of a step of
+// sequences of one length are of this kind).  Both are chains of dependent reads, so what they cost
+// is how long that chain is and how many workgroups there are to start.
+//
+// For short chunk lists (a few sequences): grid (16 rows, n_kv, max_chunks), one thread per head
+// dimension (at least one wave), a workgroup a row.  The chunks' maxima and sums are read by the first
+// wave, one chunk a lane, together with the first eight partial outputs.
+__global__ void attn_combine_rows_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    const int* __restrict__ plan, bf16_t* __restrict__ out, int out_stride,
+                                    int n_heads, int n_kv) {
+  __shared__ float f_s[COMBINE_MAX_SPLITS];  // weight of each chunk's partial output: 2^(m_s - M) / L
+  const int r = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z, d = threadIdx.x;
   const int G = n_heads / n_kv;
-  // where the partial results lie depends on the indices alone: their loads go out together with
-  // the item's, one round trip for all of them
-  const size_t row0 = (((size_t)item * n_kv + kvh) * n_splits) * 16 + r;
+  const int* rec = plan + PLAN_HEAD + (size_t)chunk * 8;
+  const int4 rec_a = *(const int4*)rec, rec_b = *(const int4*)(rec + 4);
+  const int n_splits = rec_b.z;
+  if (n_splits <= 1 || rec_b.w != 0) return;  // uniform: not in use, or written by the split kernel, or not the first
+  const Item it{rec_a.x, rec_a.y, rec_a.z, rec_a.w};
+  if (r >= it.n_tok * G) return;  // uniform: a row beyond the item, its partial results are never written
+  const size_t row0 = ((size_t)chunk * n_kv + kvh) * 16 + r, step = (size_t)n_kv * 16;  // rows from chunk to chunk
   const int dc = min(d, HD - 1);
-  float first[8];
+  float first_o[8];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) first[u] = part_o[(row0 + (size_t)min(u, n_splits - 1) * 16) * HD + dc];
-  constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
-  float ms[PER], ls[PER];
+  for (int u = 0; u < 8; ++u) first_o[u] = part_o[(row0 + (size_t)min(u, n_splits - 1) * step) * HD + dc];
   if (threadIdx.x < FG_WAVE) {
+    constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
+    float ms[PER], ls[PER];
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const int sp = threadIdx.x + j * FG_WAVE;
-      const float2 ml = *(const float2*)(part_ml + (row0 + (size_t)min(sp, n_splits - 1) * 16) * 2);
+      const float2 ml = *(const float2*)(part_ml + (row0 + (size_t)min(sp, n_splits - 1) * step) * 2);
       ms[j] = sp < n_splits ? ml.x : -INFINITY;  // maxima are in base 2
       ls[j] = ml.y;
     }
-  }
-  const Item it = load_item(items, item);
-  if (threadIdx.x < FG_WAVE) {
     float M = -INFINITY;
 #pragma unroll
     for (int j = 0; j < PER; ++j) M = fmaxf(M, ms[j]);
@@ -403,19 +506,99 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     for (int j = 0; j < PER; ++j) f_s[threadIdx.x + j * FG_WAVE] = ms[j] * inv;
   }
   __syncthreads();
-  if (d >= HD || r >= it.n_tok * G) return;  // (a row beyond the item: its partial results are never written)
+  if (d >= HD) return;
   float O = 0.f;
 #pragma unroll
-  for (int u = 0; u < 8; ++u) O += (u < n_splits ? f_s[u] : 0.f) * first[u];
+  for (int u = 0; u < 8; ++u) O += u < n_splits ? f_s[u] * first_o[u] : 0.f;
   for (int s0 = 8; s0 < n_splits; s0 += 8) {
     float v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = part_o[(row0 + (size_t)min(s0 + u, n_splits - 1) * 16) * HD + d];
+    for (int u = 0; u < 8; ++u) v[u] = part_o[(row0 + (size_t)min(s0 + u, n_splits - 1) * step) * HD + d];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) O += (s0 + u < n_splits ? f_s[s0 + u] : 0.f) * v[u];
+    for (int u = 0; u < 8; ++u) O += s0 + u < n_splits ? f_s[s0 + u] * v[u] : 0.f;
   }
   const int t = it.tok0 + r / G, h = kvh * G + r % G;
   out[(size_t)t * out_stride + (size_t)h * HD + d] = (bf16_t)O;
+}
+
+// For long chunk lists (many sequences; sixteen times fewer workgroups): grid (n_kv, max_chunks), 256
+// threads, a workgroup for the 16 rows x HD of a kv head.  Wave w weighs rows 4w .. 4w+3, one chunk a
+// lane; then every thread adds up four neighbouring head dimensions of a row (or of several rows).
+__global__ __launch_bounds__(256) void attn_combine_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ plan,
+    bf16_t* __restrict__ out, int out_stride, int n_heads, int n_kv) {
+  __shared__ float f_s[16][COMBINE_MAX_SPLITS];  // weight of each chunk's partial output: 2^(m_s - M) / L
+  const int kvh = blockIdx.x, chunk = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid % FG_WAVE, wave = tid / FG_WAVE;
+  const int G = n_heads / n_kv;
+  const int* rec = plan + PLAN_HEAD + (size_t)chunk * 8;
+  const int4 rec_a = *(const int4*)rec, rec_b = *(const int4*)(rec + 4);
+  const int n_splits = rec_b.z;
+  if (n_splits <= 1 || rec_b.w != 0) return;  // uniform: not in use, or written by the split kernel, or not the first
+  const Item it{rec_a.x, rec_a.y, rec_a.z, rec_a.w};
+  constexpr int V4 = 4 * HD;             // float4s of one chunk's 16 x HD partial output
+  constexpr int NV = (V4 + 255) / 256;   // of them a thread adds up
+  constexpr int AHEAD = 4;               // chunks whose partial outputs are requested together with the statistics
+  const size_t rows0 = ((size_t)chunk * n_kv + kvh) * 16, step = (size_t)n_kv * 16;  // rows from chunk to chunk
+  f32x4 first_o[AHEAD][NV];
+#pragma unroll
+  for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+      first_o[u][j] = *(const f32x4*)(part_o + (rows0 + (size_t)min(u, n_splits - 1) * step) * HD +
+                                      (size_t)min(tid + 256 * j, V4 - 1) * 4);
+  constexpr int PER = COMBINE_MAX_SPLITS / FG_WAVE;
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    float ms[PER], ls[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int sp = lane + j * FG_WAVE;
+      const float2 ml = *(const float2*)(part_ml + (rows0 + 4 * wave + rr + (size_t)min(sp, n_splits - 1) * step) * 2);
+      ms[j] = sp < n_splits ? ml.x : -INFINITY;  // maxima are in base 2
+      ls[j] = ml.y;
+    }
+    float M = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) M = fmaxf(M, ms[j]);
+    M = wave_max(M);
+    float L = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      ms[j] = ms[j] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[j] - M);
+      L += ms[j] * ls[j];
+    }
+    L = wave_sum(L);
+    const float inv = 1.f / L;  // (a row beyond the item's: never stored)
+#pragma unroll
+    for (int j = 0; j < PER; ++j) f_s[4 * wave + rr][lane + j * FG_WAVE] = ms[j] * inv;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int idx = tid + 256 * j;
+    if (idx >= V4) break;
+    const int r = (4 * idx) / HD, d = (4 * idx) % HD;
+    if (r >= it.n_tok * G) continue;  // a row beyond the item: its partial results are never written
+    f32x4 O = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u)
+      if (u < n_splits) O += f_s[r][u] * first_o[u][j];
+    for (int s0 = AHEAD; s0 < n_splits; s0 += 8) {
+      f32x4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = *(const f32x4*)(part_o + (rows0 + (size_t)min(s0 + u, n_splits - 1) * step) * HD + (size_t)idx * 4);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < n_splits) O += f_s[r][s0 + u] * v[u];
+    }
+    const int t = it.tok0 + r / G, h = kvh * G + r % G;
+    bf16x4 o4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o4[i] = (__bf16)O[i];
+    *(bf16x4*)(out + (size_t)t * out_stride + (size_t)h * HD + d) = o4;
+  }
 }
 
 static int page_shift_of(int page_size) {
@@ -424,27 +607,43 @@ static int page_shift_of(int page_size) {
   return -1;
 }
 
-// part_o: fp32 [n_items * n_kv * n_splits * 16 * HD], part_ml: the same rows x 2;
-// both may be null when n_splits == 1.
+// ints of a plan of max_chunks chunks
+extern "C" long long fg_attn_plan_ints(int max_chunks) { return PLAN_HEAD + 8LL * max_chunks; }
+
+// Cuts the items (int32 [n_items][4], 16-byte aligned) into chunks: see the layout of `plan` above.
+// max_chunks >= 2 * n_items; min_tiles: a chunk's tiles are a multiple of it (4: one tile a wave).
+extern "C" int fg_attn_plan(const int* items, int n_items, int window, int max_chunks, int min_tiles, int* plan,
+                            hipStream_t stream) {
+  if (n_items <= 0) return FG_OK;
+  if (!items || !plan || max_chunks < 2 * n_items || min_tiles < 1 || window < 0) return FG_ERR_ARG;
+  attn_plan_kernel<<<1, 256, 0, stream>>>(items, n_items, window, max_chunks, min_tiles, plan);
+  return fg_launch_status();
+}
+
+// plan: what fg_attn_plan made of the items, with the same n_items, max_chunks and window.
+// part_o: fp32 [max_chunks * n_kv * 16 * HD], part_ml: the same rows x 2.
 extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
-                             const void* v_pages, const int* block_table, int bt_stride, const int* items,
-                             int n_items, float* part_o, float* part_ml, int n_splits, int n_heads, int n_kv,
+                             const void* v_pages, const int* block_table, int bt_stride, const int* plan,
+                             int n_items, int max_chunks, float* part_o, float* part_ml, int n_heads, int n_kv,
                              int hd, int page_size, float scale, int window, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
-      !(scale > 0.f) || n_splits < 1 || n_splits > COMBINE_MAX_SPLITS || n_kv > 65535 || n_items > 65535 || window < 0 || q_stride % 8 ||
-      out_stride % 4 || (n_splits > 1 && (!part_o || !part_ml)))
+      !(scale > 0.f) || max_chunks < 2 * n_items || max_chunks > 65535 || n_kv > 65535 || window < 0 ||
+      q_stride % 8 || out_stride % 4 || !plan || !part_o || !part_ml)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                           \
-  attn_split_kernel<PERM><<<dim3(n_splits, n_kv, n_items), 256, 0, stream>>>(                                  \
+  attn_split_kernel<PERM><<<dim3(n_kv, max_chunks), 256, 0, stream>>>(                                         \
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,    \
-      block_table, bt_stride, items, part_o, part_ml, n_heads, n_kv, page_size, page_shift_of(page_size), scale, \
-      window)
+      block_table, bt_stride, plan, part_o, part_ml, n_heads, n_kv, page_size,                                 \
+      page_shift_of(page_size), scale, window)
   if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
 #undef LAUNCH
-  if (n_splits > 1)
-    attn_combine_kernel<<<dim3(16, n_kv, n_items), HD < 64 ? 64 : HD, 0, stream>>>(
-        part_o, part_ml, items, (bf16_t*)out, out_stride, n_heads, n_kv, n_splits);
+  if ((long long)max_chunks * n_kv * 16 <= COMBINE_ROWS_MAX_GROUPS)
+    attn_combine_rows_kernel<<<dim3(16, n_kv, max_chunks), HD < 64 ? 64 : HD, 0, stream>>>(
+        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
+  else
+    attn_combine_kernel<<<dim3(n_kv, max_chunks), 256, 0, stream>>>(
+        part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
   return fg_launch_status();
 }
 

@@ -283,14 +283,45 @@ def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int =
     return as_arr(small), as_arr(big)
 
 
+def attention_chunks_for(n_items: int, n_kv: int) -> int:
+    """Length of the split kernel's chunk list for ``n_items`` items: enough chunks for a few
+    workgroups per compute unit, and at least two an item so that a long sequence among short
+    ones can be cut."""
+    return max(-(-_SPLIT_TARGET_BLOCKS // n_kv) + n_items, 2 * n_items)
+
+
+def _plan_ints(lib, max_chunks: int) -> int:
+    lib.fg_attn_plan_ints.restype = ctypes.c_longlong
+    return int(lib.fg_attn_plan_ints(max_chunks))
+
+
+def attention_plan(items: torch.Tensor, n_items: int, max_chunks: int, head_dim: int, window: int = 0,
+                   min_tiles: int = 4) -> torch.Tensor:
+    """Cuts the key ranges of ``items`` (device int32 ``[n_items, 4]``, 16-byte aligned) into chunks of
+    the same number of 64-key tiles, a multiple of ``min_tiles``, on the device: a captured step cuts
+    anew for the lengths of every replay.  The int32 plan that :func:`paged_attention_mfma` takes."""
+    _gpu(items)
+    _i32(items, "items")
+    _need(items.data_ptr() % 16 == 0 and items.numel() >= 4 * n_items > 0, "items must be [n, 4], 16-byte aligned")
+    _need(max_chunks >= 2 * n_items and min_tiles >= 1, "max_chunks must be at least twice the number of items")
+    lib = _lib.load(f"attention_mfma@{head_dim}")  # the plan is the same for every head size
+    plan = torch.empty(_plan_ints(lib, max_chunks), dtype=torch.int32, device=items.device)
+    _check(lib.fg_attn_plan(_ptr(items), n_items, int(window or 0), max_chunks, min_tiles, _ptr(plan),
+                            _stream(items)), "attn_plan")
+    return plan
+
+
 def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
-                         n_splits: int = 1) -> torch.Tensor:
+                         plan: Optional[torch.Tensor] = None, max_chunks: Optional[int] = None,
+                         min_tiles: int = 4) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
     device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
-    every query token of the step must be covered by exactly one item."""
-    _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items)
+    every query token of the step must be covered by exactly one item.
+    ``plan``: :func:`attention_plan` of the small items with this ``max_chunks``
+    and ``window`` (made here if not given)."""
+    _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
           and v_pages.dtype == torch.bfloat16, "the MFMA attention kernels take bfloat16")
@@ -312,19 +343,20 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
         _i32(small_items, "small_items")
         _need(small_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
         n = small_items.numel() // 4
-        part_o = part_ml = None
-        if n_splits > 1:
-            part_o = torch.empty((n * n_kv * n_splits * 16, hd), dtype=torch.float32, device=q.device)
-            part_ml = torch.empty((n * n_kv * n_splits * 16, 2), dtype=torch.float32, device=q.device)
-        for i0 in range(0, n, 65535):  # grid.z limit
-            ni = min(65535, n - i0)
-            st = lib.fg_attn_split(
-                _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-                block_table.stride(0), ctypes.c_void_p(small_items.data_ptr() + 16 * i0), ni,
-                ctypes.c_void_p(part_o.data_ptr() + 4 * i0 * n_kv * n_splits * 16 * hd if part_o is not None else 0),
-                ctypes.c_void_p(part_ml.data_ptr() + 4 * i0 * n_kv * n_splits * 16 * 2 if part_ml is not None else 0),
-                n_splits, n_heads, n_kv, hd, page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
-            _check(st, "attn_split")
+        if max_chunks is None:
+            max_chunks = attention_chunks_for(n, n_kv)
+        _need(2 * n <= max_chunks <= 65535, "the chunk list holds at least two chunks an item and at most 65535")
+        if plan is None:
+            plan = attention_plan(small_items, n, max_chunks, hd, window, min_tiles)
+        _need(plan.dtype == torch.int32 and plan.numel() == _plan_ints(lib, max_chunks),
+              "the plan does not fit the items and max_chunks")
+        part_o = torch.empty((max_chunks * n_kv * 16, hd), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((max_chunks * n_kv * 16, 2), dtype=torch.float32, device=q.device)
+        st = lib.fg_attn_split(
+            _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+            block_table.stride(0), _ptr(plan), n, max_chunks, _ptr(part_o), _ptr(part_ml), n_heads, n_kv, hd,
+            page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
+        _check(st, "attn_split")
     if big_items is not None and big_items.numel():
         _need(G <= attention_tile_rows(hd), "too many query heads per kv head for the tile kernel")
         _i32(big_items, "big_items")
@@ -364,12 +396,16 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
             plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small))
         ctx.scratch[("attention_items", G)] = plan
     small_d, big_d, n_small = plan
-    n_splits = 1
+    chunks = split_plan = None
     if n_small:
-        tiles = -(-(ctx.graph_capacity or ctx.max_kv_len) // 64)
-        n_splits = max(1, min(-(-tiles // 4), -(-_SPLIT_TARGET_BLOCKS // (n_small * n_kv)), 64))
+        # how the items' key ranges are cut depends on the window: layers with the same one share the cut
+        chunks = attention_chunks_for(n_small, n_kv)
+        key = ("attention_plan", G, int(window or 0), chunks)
+        split_plan = ctx.scratch.get(key)
+        if split_plan is None:
+            split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window)
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
-                                window, n_splits)
+                                window, split_plan, chunks)
 
 
 # ----------------------------------------------------------------------- gemm

@@ -515,7 +515,12 @@ def test_kernels_refuse_what_they_cannot_take(ops):
 
 
 # ------------------------------------------------------- attention on MFMA
-def _run_mfma(ops, case, seqs, H, KV, window=0, n_splits=1):
+# how the split kernel's key ranges are cut: (max_chunks, min_tiles); max_chunks None: the engine's
+# choice, "least": twice the items (the fewest chunks), a large number with min_tiles 1: one tile a chunk
+CUTS = {"auto": (None, 4), "coarse": ("least", 4), "fine": (4096, 1), "pairs": (4096, 2)}
+
+
+def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto"):
     import numpy as np
 
     q_lens = [b for _, b in seqs]
@@ -524,8 +529,11 @@ def _run_mfma(ops, case, seqs, H, KV, window=0, n_splits=1):
                                      ops.attention_tile_rows(case["kp"].shape[3]))
     dev = lambda a: torch.from_numpy(a.reshape(-1)).to(DEV) if a.size else None
     out = torch.full_like(case["q"], float("nan"))
+    max_chunks, min_tiles = CUTS[cut]
+    if max_chunks == "least":
+        max_chunks = 2 * len(small)
     ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], dev(small), dev(big), H,
-                             case["kp"].shape[3] ** -0.5, window, n_splits)
+                             case["kp"].shape[3] ** -0.5, window, None, max_chunks, min_tiles)
     return out, len(small), len(big)
 
 
@@ -545,26 +553,26 @@ MFMA_SEQS = [(0, 1), (0, 70), (131, 1), (60, 9), (17, 2), (255, 1), (0, 129), (3
 
 @pytest.mark.parametrize("H,KV,hd,P", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37, 150])
-@pytest.mark.parametrize("n_splits", [1, 3])
-def test_paged_attention_mfma(ops, H, KV, hd, P, window, n_splits):
+@pytest.mark.parametrize("cut", ["coarse", "fine"])
+def test_paged_attention_mfma(ops, H, KV, hd, P, window, cut):
     case = _paged_case(torch.bfloat16, MFMA_SEQS, H, KV, hd, P, seed=21)
-    out, n_small, n_big = _run_mfma(ops, case, MFMA_SEQS, H, KV, window, n_splits)
+    out, n_small, n_big = _run_mfma(ops, case, MFMA_SEQS, H, KV, window, cut)
     assert n_small and n_big  # both kernels run
     want = _plain_rows(case, MFMA_SEQS, window or None)
     assert torch.isfinite(out).all()  # every row written, no poison read
     assert torch.allclose(out.cpu().float(), want, atol=1.5e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("n_splits", [1, 2, 8])
-def test_paged_attention_mfma_far_key_and_edges(ops, n_splits):
+@pytest.mark.parametrize("cut", ["coarse", "pairs", "fine"])
+def test_paged_attention_mfma_far_key_and_edges(ops, cut):
     """A key that gets nearly all the weight, at the edges of tiles, pages and
-    splits, for a decoded token (split kernel) and inside a portion (tile
+    chunks, for a decoded token (split kernel) and inside a portion (tile
     kernel)."""
     H, KV, hd, P = 8, 2, 64, 16
     for kpos in (0, 15, 16, 63, 64, 127, 128, 300, 399, 400):
         for seqs, qpos, row in (([(0, 3), (400, 1), (10, 2)], 400, 3), ([(0, 2), (380, 40)], 400, 2 + 20)):
             case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=22, peak=(1, qpos, 5, kpos))
-            out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, n_splits)
+            out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, cut)
             v = case["whole"][2][1]
             got = out.cpu().float()[row].view(H, hd)[5]
             assert torch.allclose(got, v[kpos, 1].float(), atol=2e-2), (kpos, seqs)
@@ -576,20 +584,62 @@ def test_paged_attention_mfma_window_edge(ops):
     for seqs, row in (([(100, 1)], 0), ([(90, 30)], 10)):
         for kpos, seen in ((100 - w, False), (100 - w + 1, True)):
             case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=23, peak=(0, 100, 1, kpos))
-            out, _, _ = _run_mfma(ops, case, seqs, H, KV, w, 2)
+            out, _, _ = _run_mfma(ops, case, seqs, H, KV, w, "fine")
             v = case["whole"][2][0]
             got = out.cpu().float()[row].view(H, hd)[1]
             assert torch.allclose(got, v[kpos, 0].float(), atol=2e-2) == seen
             assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs, w), atol=1.5e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("n_splits", [16, 64, 200])
-def test_paged_attention_mfma_long_context(ops, n_splits):
+@pytest.mark.parametrize("cut,longest", [("auto", 5000), ("fine", 5000), ("fine", 17000), ("coarse", 5000)])
+def test_paged_attention_mfma_long_context(ops, cut, longest):
     """Llama-3.1-8B's attention shape at a context of several thousand keys,
-    one decoded token and one long portion; with more splits than one wave
-    of the combine has lanes, and more splits than the short sequence has tiles."""
+    one decoded token and one long portion, beside a short sequence that has
+    one chunk; with more chunks an item than one wave of the combine has
+    lanes, and (17,000 keys, one tile a chunk asked for) more tiles than an
+    item may have chunks."""
     H, KV, hd, P = 32, 8, 128, 64
-    seqs = [(5000, 1), (3000, 200), (70, 1)]
+    seqs = [(longest, 1), (3000, 200), (70, 1)]
     case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=24, poison=True)
-    out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, n_splits)
+    out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, cut)
     assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("n_items,window,max_chunks,min_tiles", [
+    (1, 0, 2, 4), (7, 0, 128, 4), (7, 100, 14, 1), (300, 0, 600, 4), (300, 777, 1024, 1), (513, 0, 4096, 2),
+])
+def test_attention_plan_cuts_every_item_into_equal_chunks(ops, n_items, window, max_chunks, min_tiles):
+    """The plan that the split kernel works from: every item's tiles are covered once, in order, by
+    chunks of the plan's size (the last may be shorter), the items' chunks one after the other; no
+    more chunks than the list holds, none in use beyond the count, at most 256 an item."""
+    import numpy as np
+
+    rng = np.random.default_rng(n_items + window)
+    n_tok = rng.integers(1, 4, n_items)
+    pos0 = rng.integers(0, 40000 if n_items < 10 else 6000, n_items)
+    items = np.stack([np.arange(n_items), np.cumsum(n_tok) - n_tok, n_tok, pos0], axis=1).astype(np.int32)
+    plan = ops.attention_plan(torch.from_numpy(items.reshape(-1)).to(DEV), n_items, max_chunks, 128, window,
+                              min_tiles).cpu().numpy()
+    ts, used = int(plan[0]), int(plan[1])
+    chunks = plan[4: 4 + 8 * max_chunks].reshape(max_chunks, 8)
+    assert ts % min_tiles == 0 and 0 < used <= max_chunks
+    assert (chunks[used:, 6] == 0).all() and (chunks[:used, 6] > 0).all()
+    nxt = 0
+    for i in range(n_items):
+        last = pos0[i] + n_tok[i] - 1
+        first_key = max(0, pos0[i] - window + 1) if window else 0
+        t_lo, t_hi = first_key // 64, last // 64
+        count = -(-(t_hi - t_lo + 1) // ts)
+        assert count <= 256
+        for c in range(count):
+            rec = chunks[nxt + c]
+            assert tuple(rec[:4]) == tuple(items[i]) and rec[6] == count and rec[7] == c
+            assert rec[4] == t_lo + c * ts and rec[5] == min(t_hi + 1, t_lo + (c + 1) * ts)
+        nxt += count
+    assert nxt == used
+    # coarser is never needed: with chunks one step smaller the list would overflow, or it is the least allowed
+    if ts > min_tiles:
+        smaller = ts - min_tiles
+        tiles = [(pos0[i] + n_tok[i] - 1) // 64 - ((max(0, pos0[i] - window + 1) if window else 0) // 64) + 1
+                 for i in range(n_items)]
+        assert sum(tiles) / smaller + n_items > max_chunks or max(tiles) > 256 * smaller
