@@ -253,6 +253,8 @@ MFMA_MAX_HEAD_DIM = 256
 # them in the split that finishes last needs device-scope fences, which on a GPU of several
 # dies cost more than the launch they save (measured).
 _SPLIT_TARGET_BLOCKS = int(os.environ.get("FG_SPLIT_TARGET", 256))
+# a chunk of the decode attention's key ranges is a multiple of this many 64-key tiles (one a wave)
+_SPLIT_MIN_TILES = int(os.environ.get("FG_SPLIT_MIN_TILES", 4))
 
 
 def attention_tile_rows(head_dim: int) -> int:
@@ -403,7 +405,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
         key = ("attention_plan", G, int(window or 0), chunks)
         split_plan = ctx.scratch.get(key)
         if split_plan is None:
-            split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window)
+            split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window, _SPLIT_MIN_TILES)
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
                                 window, split_plan, chunks)
 

@@ -101,11 +101,16 @@ def test_token_by_token_from_the_first(case, dtype):
     assert_close(got, {rid: case["want"][rid]}, dtype, case["noise"], "one-by-one")
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_long_decoding_of_a_batch(dtype, tmp_path):
+@pytest.mark.parametrize("dtype,min_tiles", [(torch.float32, 4), (torch.bfloat16, 4), (torch.bfloat16, 1)])
+def test_long_decoding_of_a_batch(dtype, min_tiles, tmp_path, monkeypatch):
     """Three requests decode together for hundreds of steps (the captured decode
-    step is replayed while block tables grow over dozens of small pages and the
-    requests end one after the other), every position against the plain run."""
+    step is replayed while block tables grow over dozens of small pages, the
+    requests' key ranges are cut into more and more chunks, of four tiles and
+    of one, and the requests end one after the other), every position against
+    the plain run."""
+    from fastgen_amd.kernels import ops
+
+    monkeypatch.setattr(ops, "_SPLIT_MIN_TILES", min_tiles)
     cfg = TINY_C
     weights = sharpen(plain_random_weights(cfg, 7))
     weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
