@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
+from ..kernels.ops import upload
 
 
 @dataclass
@@ -26,6 +27,9 @@ class StepEntry:
     rid: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # the entry's one token is row ``from_row`` of the tokens that the step before sampled and the
+    # host has not seen (the step function is given that tensor); ``tokens`` then holds a stand-in
+    from_row: Optional[int] = None
 
 
 @dataclass
@@ -157,5 +161,5 @@ def build_context(entries: Sequence[StepEntry], cache: CacheManager, act_dtype: 
     """Host vectors for ``entries`` (whose pages are already reserved), packed
     into one int32 buffer and copied to the device once."""
     packed, offs, table_shapes, host = pack_context(entries, cache, vocab_size)
-    return context_from_packed(torch.from_numpy(packed).to(device), offs, table_shapes, host, cache.page_size,
+    return context_from_packed(upload(packed, torch.int32, device), offs, table_shapes, host, cache.page_size,
                                act_dtype)

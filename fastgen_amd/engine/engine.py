@@ -7,7 +7,9 @@ interface on top of this class.)
 
 from __future__ import annotations
 
+import os
 import time
+from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Dict, Hashable, Iterable, List, Mapping, Optional, Sequence
 
@@ -17,13 +19,25 @@ from ..sampling import Sampler, SamplingParams
 from .context import StepEntry
 from .model import Model
 from .runner import ModelRunner
-from .scheduler import PlannedEntry, Request, Scheduler
+from .scheduler import PENDING, PlannedEntry, Request, Scheduler
+
+
+@dataclass
+class _InFlight:
+    """A step whose samples the host has not seen yet."""
+
+    plan: List[PlannedEntry]
+    tokens: torch.Tensor  # int32 [rows] on the device: what the next step's entries take their tokens from
+    row_of: Dict[int, int]  # id(request) -> its row
+    host_tokens: torch.Tensor  # pinned copy, complete once ``copied`` has happened
+    host_logprobs: Optional[torch.Tensor]
+    copied: torch.cuda.Event
 
 
 class Engine:
     def __init__(self, model: Model, page_size: int = 64, max_tokens: int = 8192, max_batch: int = 64,
                  max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0,
-                 sync_freq: int = 10) -> None:
+                 sync_freq: int = 10, overlap_steps: Optional[bool] = None) -> None:
         self.model = model
         self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch)
         cap = getattr(model.args, "max_position", 0) or None
@@ -39,6 +53,15 @@ class Engine:
         # decode steps between host checks for finished requests when nothing waits for admission
         # (the reference's GenArgs.sync_freq, fastgen/generate.py:55-59)
         self.sync_freq = sync_freq
+        # The host runs one step behind the device: a step is planned and launched from the counts of
+        # tokens alone, the step before it hands its samples over on the device, and the host looks
+        # at them (stop ids, the caller's lists) while the new step runs.  FG_NO_OVERLAP=1 (or False
+        # here) makes every step wait for its tokens.
+        if overlap_steps is None:
+            overlap_steps = os.environ.get("FG_NO_OVERLAP", "0") in ("", "0")
+        self.overlap_steps = overlap_steps
+        self._in_flight: Optional[_InFlight] = None
+        self._held: List[Request] = []  # ended, with samples still on the device
         self._n_requests = 0
         self.n_steps = 0
 
@@ -72,7 +95,7 @@ class Engine:
         return rid
 
     def has_work(self) -> bool:
-        return self.scheduler.has_work()
+        return self.scheduler.has_work() or self._in_flight is not None or bool(self._held)
 
     def abort(self, rid: Hashable) -> bool:
         """End a request before it is done; it comes out of the next ``step`` with ``finish_reason``
@@ -81,42 +104,89 @@ class Engine:
 
     def step(self) -> List[Request]:
         """One step of the model over what the scheduler picks; the requests
-        that ended with it."""
-        n_run = self.scheduler.plan_decode_run(self.sync_freq) if self.runner.can_graph(len(self.scheduler.running)) else 0
-        if n_run:
-            return self._ended(self._decode_run(n_run))
-        plan = self.scheduler.plan()
-        done: List[Request] = []
-        if plan:
-            entries, rows = [], []
-            for e in plan:
-                toks = e.request.tokens_from(e.start, e.n)
-                entries.append(StepEntry(e.request.rid, toks, [e.n - 1] if e.wants_logits else []))
-                if e.wants_logits:
-                    rows.append(e.request)
-            logits = self.runner.step(entries)
-            sampled: List[int] = []
-            lps = None
-            if rows:
-                tok = self.sampler.sample(
-                    logits, [r.temperature for r in rows], [r.top_p for r in rows], [r.seed for r in rows],
-                    [len(r.generated) for r in rows],
-                )
-                if any(r.want_logprobs for r in rows):
-                    lps = self.sampler.logprobs(logits, tok).tolist()
-                sampled = tok.tolist()
-            done = self.scheduler.commit(plan, sampled, lps)
-            self.n_steps += 1
+        that ended and whose tokens the host has all seen (with overlapped steps
+        a request is reported a step after its last one)."""
+        sched = self.scheduler
+        if self.runner.can_graph(len(sched.running)):
+            if self._in_flight is not None and self._decode_run_ahead():
+                self._settle()  # a decode run starts from tokens the host knows; a stop id among them may end one
+            n_run = sched.plan_decode_run(self.sync_freq)
+            if n_run:
+                return self._ended(self._decode_run(n_run))
+        plan = sched.plan()
+        if not plan:
+            self._settle()
+            return self._ended([])
+        entries, rows = [], []
+        prev = self._in_flight
+        for e in plan:
+            toks = e.request.tokens_from(e.start, e.n)
+            from_row = None
+            if PENDING in toks:
+                if e.n != 1 or prev is None:  # only ever the one token of a decoding request
+                    raise RuntimeError(f"request {e.request.rid!r}: a portion holds a token the host has not seen")
+                from_row, toks = prev.row_of[id(e.request)], [0]
+            entries.append(StepEntry(e.request.rid, toks, [e.n - 1] if e.wants_logits else [], from_row))
+            if e.wants_logits:
+                rows.append(e.request)
+        logits = self.runner.step(entries, prev.tokens if prev is not None else None)
+        self.n_steps += 1
+        tok = lps = None
+        if rows:
+            tok = self.sampler.sample(
+                logits, [r.temperature for r in rows], [r.top_p for r in rows], [r.seed for r in rows],
+                [len(r.generated) for r in rows],
+            )
+            if any(r.want_logprobs for r in rows):
+                lps = self.sampler.logprobs(logits, tok)
+        if not rows:  # portions of prompts only: nothing to wait for
+            done = sched.commit(plan, [])
+            self._settle()
+            return self._ended(done)
+        if not self.overlap_steps:
+            done = sched.commit(plan, tok.tolist(), lps.tolist() if lps is not None else None)
+            return self._ended(done)
+        host_tok = torch.empty(tok.shape, dtype=tok.dtype, pin_memory=True)
+        host_tok.copy_(tok, non_blocking=True)
+        host_lps = None
+        if lps is not None:
+            host_lps = torch.empty(lps.shape, dtype=lps.dtype, pin_memory=True)
+            host_lps.copy_(lps, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        done = sched.commit(plan)  # its samples stay on the device for now
+        self._in_flight = _InFlight(plan, tok, {id(r): i for i, r in enumerate(rows)}, host_tok, host_lps, copied)
+        if prev is not None:
+            self._resolve(prev)  # the step before: its tokens have long arrived
         return self._ended(done)
+
+    def _decode_run_ahead(self) -> bool:
+        """Whether a decode run would start once the step in flight is settled."""
+        sched = self.scheduler
+        return bool(sched.running) and not sched.waiting and all(r.remaining() == 1 for r in sched.running)
+
+    def _resolve(self, step: _InFlight) -> None:
+        step.copied.synchronize()
+        self.scheduler.resolve(step.plan, step.host_tokens.tolist(),
+                               step.host_logprobs.tolist() if step.host_logprobs is not None else None)
+
+    def _settle(self) -> None:
+        """Wait for the samples of the step in flight and let the scheduler see them."""
+        if self._in_flight is not None:
+            step, self._in_flight = self._in_flight, None
+            self._resolve(step)
 
     def _ended(self, done: List[Request]) -> List[Request]:
         """``done`` and what else the scheduler ended since the last step (a request alone and out
-        of pages ends while planning); every ended request is reported once."""
-        for r in self.scheduler.finished:
-            if r not in done:
-                done.append(r)
+        of pages ends while planning, a stop id ends one a step late); every ended request is
+        reported once, when the host has seen all its tokens."""
+        for r in done + self.scheduler.finished:
+            if not any(r is h for h in self._held):
+                self._held.append(r)
         self.scheduler.finished.clear()
-        return done
+        out = [r for r in self._held if r.n_pending == 0]
+        self._held = [r for r in self._held if r.n_pending]
+        return out
 
     def _decode_run(self, n_steps: int) -> List[Request]:
         """``n_steps`` decode steps of all running requests with one look at the
@@ -208,5 +278,7 @@ class Engine:
         dt = time.perf_counter() - t0
         for r in list(self.scheduler.running):  # the measurement is over: let go of the batch
             self.abort(r.rid)
+        self._settle()
         self.scheduler.finished.clear()
+        self._held.clear()
         return dt

@@ -18,6 +18,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..cache.storage import CacheStorage, group_entries
+from ..kernels.ops import upload
 from .context import StepContext, StepEntry, build_context, context_from_packed, pack_context
 from .model import Model
 
@@ -165,20 +166,44 @@ class ModelRunner:
             self.cache.reserve(e.rid, len(e.tokens))
         return build_context(entries, self.cache, self.model.dtype, self.model.device, self.model.vocab_size)
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], prev_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """fp32 logits ``[n_wanted, vocab]`` in the order of the entries and
         of their ``want`` lists; None if nothing is wanted.  The tensor may be
         the buffer of a captured step: it holds these logits until the next
-        step; copy what is to be kept."""
+        step; copy what is to be kept.  ``prev_tokens``: int32 tokens on the
+        device that entries with ``from_row`` take their token from."""
+        fill = self._token_fill(entries, prev_tokens)
         if self.use_graphs and self._is_plain_decode(entries):
-            logits = self._graph_step(entries)
+            logits = self._graph_step(entries, fill)
         else:
             ctx = self.prepare(entries)
             self.last_context = ctx
+            if fill is not None:
+                ctx.tokens.index_copy_(0, fill[0], fill[1])
             logits = self.model.forward(ctx, self.stores)
         for e in entries:
             self.cache.advance(e.rid, len(e.tokens))
         return logits
+
+    def _token_fill(self, entries: Sequence[StepEntry], prev_tokens: Optional[torch.Tensor]):
+        """(flat token indices, their tokens) on the device for the entries whose token is still
+        there, or None."""
+        dst, src, at = [], [], 0
+        for e in entries:
+            if e.from_row is not None:
+                if len(e.tokens) != 1:
+                    raise ValueError(f"request {e.rid!r}: only a single token can come from the step before")
+                dst.append(at)
+                src.append(e.from_row)
+            at += len(e.tokens)
+        if not dst:
+            return None
+        if prev_tokens is None or prev_tokens.dtype != torch.int32:
+            raise ValueError("entries name rows of the last step's tokens: give them as an int32 tensor")
+        if max(src) >= prev_tokens.numel():
+            raise ValueError("an entry names a row beyond the last step's tokens")
+        idx = upload([dst, src], torch.int64, self.model.device)
+        return idx[0], prev_tokens.index_select(0, idx[1])
 
     # ------------------------------------------------------- decode graphs
     def _is_plain_decode(self, entries: Sequence[StepEntry]) -> bool:
@@ -227,10 +252,14 @@ class ModelRunner:
                 self.cache.advance(e.rid, 1)
         return out
 
-    def _graph_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _graph_step(self, entries: Sequence[StepEntry], fill=None) -> torch.Tensor:
         if len({e.rid for e in entries}) != len(entries):
             raise ValueError("a request appears twice in one step")
         for e in entries:
             self.cache.reserve(e.rid, 1)
+        tokens = None
+        if fill is not None:  # some tokens are on the device: the replay takes all of them from there
+            tokens = upload([e.tokens[0] for e in entries], torch.int32, self.model.device)
+            tokens.index_copy_(0, fill[0], fill[1])
         # (a capture runs the step's kernels only as a recording: the replay gives this step's result)
-        return self._graph_for(entries).replay(self, entries)
+        return self._graph_for(entries).replay(self, entries, tokens)

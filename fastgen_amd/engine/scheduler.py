@@ -19,6 +19,11 @@ portions in arrival order, so prompt portions ride beside decoded tokens.
   length cap, ``509-513``).
 * A request ends when it samples a stop id, has ``max_new`` tokens, or reaches
   ``max_seq`` tokens (``95-113``, ``445-447``, ``637-662``).
+* The host may run one step behind the device: ``commit`` without tokens records
+  a step whose samples are still on the device (a ``PENDING`` place in
+  ``generated``), the next plan is made from the counts alone, and ``resolve``
+  fills the values in when they arrive.  A stop id then ends its request one step
+  late: what the request did in that step is dropped.
 """
 
 from __future__ import annotations
@@ -28,6 +33,9 @@ from dataclasses import dataclass, field
 from typing import Callable, Deque, Hashable, List, Optional, Sequence, Tuple
 
 from ..cache.manager import CacheManager
+
+
+PENDING = -1  # in ``Request.generated``: a token that the device has sampled and the host has not seen yet
 
 
 @dataclass(eq=False)  # requests are compared by identity: two with equal fields are still two
@@ -43,6 +51,7 @@ class Request:
     generated: List[int] = field(default_factory=list)
     logprobs: List[float] = field(default_factory=list)
     n_fed: int = 0  # tokens of prompt + generated whose keys are in the cache
+    n_pending: int = 0  # PENDING places in ``generated``
     preemptions: int = 0
     finish_reason: Optional[str] = None
 
@@ -73,6 +82,7 @@ class PlannedEntry:
     start: int  # index into all_tokens()
     n: int
     wants_logits: bool  # this portion ends at the last known token
+    gen_index: int = -1  # where in ``generated`` the step's sample goes (set by ``commit``)
 
 
 class Scheduler:
@@ -190,6 +200,8 @@ class Scheduler:
         # C. admission: preempted requests first (they sit at the head), then new ones
         while self.waiting and len(self.running) < self.max_batch and budget > 0:
             req = self.waiting[0]
+            if req.n_pending:  # preempted in this very plan with a sample still on the device: next time
+                break
             need = req.n_known() + 1
             if any(self.cache.pages_needed_fresh(need, g) > self.cache.free_pages(g)
                    for g in range(self.cache.n_groups)):
@@ -220,7 +232,7 @@ class Scheduler:
             return 0
         n = max_steps
         for req in self.running:
-            if req.remaining() != 1:
+            if req.remaining() != 1 or req.n_pending:
                 return 0
             n = min(n, req.max_new - len(req.generated), self.max_seq - req.n_known())
         if n < 2:
@@ -260,30 +272,77 @@ class Scheduler:
         return done
 
     # ------------------------------------------------------------- commit
-    def commit(self, entries: Sequence[PlannedEntry], sampled: Sequence[int],
+    def commit(self, entries: Sequence[PlannedEntry], sampled: Optional[Sequence[int]] = None,
                logprobs: Optional[Sequence[float]] = None) -> List[Request]:
         """Record what the step did: ``sampled`` holds one token for every
-        entry that wanted logits, in order.  Returns the requests that ended."""
+        entry that wanted logits, in order.  Returns the requests that ended.
+
+        With ``sampled`` None the samples are still on the device: the places
+        in ``generated`` are marked ``PENDING`` (and :meth:`resolve` fills them
+        in), and only what does not depend on a token's value ends a request
+        here (its count of tokens, its length)."""
         done: List[Request] = []
-        it = iter(range(len(sampled)))
+        i = -1
         for e in entries:
             req = e.request
             req.n_fed += e.n
             if not e.wants_logits:
                 continue
-            i = next(it)
-            tok = int(sampled[i])
-            req.generated.append(tok)
-            if logprobs is not None and req.want_logprobs:
-                req.logprobs.append(float(logprobs[i]))
-            if tok in req.stop_ids:
-                reason = "stop"
-            elif len(req.generated) >= req.max_new:
-                reason = "length"
-            elif req.n_known() >= self.max_seq:
-                reason = "max_seq"
+            i += 1
+            e.gen_index = len(req.generated)
+            reason = None
+            if sampled is None:
+                req.generated.append(PENDING)
+                req.n_pending += 1
+                if req.want_logprobs:
+                    req.logprobs.append(0.0)
             else:
-                continue
-            self._finish(req, reason)
-            done.append(req)
+                tok = int(sampled[i])
+                req.generated.append(tok)
+                if logprobs is not None and req.want_logprobs:
+                    req.logprobs.append(float(logprobs[i]))
+                if tok in req.stop_ids:
+                    reason = "stop"
+            if reason is None:
+                if len(req.generated) >= req.max_new:
+                    reason = "length"
+                elif req.n_known() >= self.max_seq:
+                    reason = "max_seq"
+            if reason:
+                self._finish(req, reason)
+                done.append(req)
         return done
+
+    def resolve(self, entries: Sequence[PlannedEntry], sampled: Sequence[int],
+                logprobs: Optional[Sequence[float]] = None) -> List[Request]:
+        """The tokens of a step that was committed without them have arrived.
+        A request that sampled a stop id ends there: what it generated after
+        that token (a later step may be committed already) is dropped.  Returns
+        the requests that this ended."""
+        late: List[Request] = []
+        i = -1
+        for e in entries:
+            if not e.wants_logits:
+                continue
+            i += 1
+            req = e.request
+            if e.gen_index >= len(req.generated):
+                continue  # dropped: the request ended on an earlier token
+            if req.generated[e.gen_index] != PENDING:
+                raise RuntimeError(f"request {req.rid!r}: token {e.gen_index} resolved twice")
+            tok = int(sampled[i])
+            req.generated[e.gen_index] = tok
+            req.n_pending -= 1
+            if logprobs is not None and req.want_logprobs:
+                req.logprobs[e.gen_index] = float(logprobs[i])
+            if tok in req.stop_ids and req.finish_reason != "aborted":
+                dropped = req.generated[e.gen_index + 1:]
+                req.n_pending -= sum(1 for t in dropped if t == PENDING)
+                del req.generated[e.gen_index + 1:]
+                del req.logprobs[e.gen_index + 1:]
+                if req.finish_reason is None:
+                    self._finish(req, "stop")
+                    late.append(req)
+                else:  # its count of tokens had ended it already: the stop id is the reason
+                    req.finish_reason = "stop"
+        return late

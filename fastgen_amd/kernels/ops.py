@@ -56,6 +56,19 @@ def _stream(t: torch.Tensor) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
+def upload(values, dtype: torch.dtype, device: torch.device | str) -> torch.Tensor:
+    """``values`` (a numpy array or nested lists) on the device, through pinned host memory and a
+    copy that does not make the host wait for the work already queued on the stream: a step can be
+    prepared while the step before it runs.  (The pinned block goes back to torch's host allocator,
+    which hands it out again only after the copy has happened.)"""
+    src = torch.from_numpy(values) if isinstance(values, np.ndarray) else torch.tensor(values, dtype=dtype)
+    if src.dtype != dtype:
+        src = src.to(dtype)
+    staged = torch.empty(src.shape, dtype=dtype, pin_memory=True)
+    staged.copy_(src)
+    return staged.to(device, non_blocking=True)
+
+
 def _check(status: int, what: str) -> None:
     if status == 1:
         raise KernelArgumentError(f"{what}: the kernel refuses these sizes or dtypes")
@@ -394,7 +407,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
             plan = (ctx.seq_records, None, ctx.n_seqs)
         else:
             small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, attention_tile_rows(hd))
-            both = torch.from_numpy(np.concatenate([small, big]).reshape(-1)).to(q.device)
+            both = upload(np.concatenate([small, big]).reshape(-1), torch.int32, q.device)
             plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small))
         ctx.scratch[("attention_items", G)] = plan
     small_d, big_d, n_small = plan

@@ -48,10 +48,10 @@ class Sampler:
         counter at step ``s`` is ``counters[row] + s``."""
         if not any(t > 0 for t in temperatures):
             return lambda logits, step, out: ops.sample(logits, out=out)
-        packed_f = torch.tensor([list(temperatures), list(top_ps)], dtype=torch.float32).to(self.device)
+        packed_f = ops.upload([list(temperatures), list(top_ps)], torch.float32, self.device)
         mask = (1 << 63) - 1
         ints = [[s & mask for s in seeds]] + [[c + s for c in counters] for s in range(n_steps)]
-        packed_i = torch.tensor(ints, dtype=torch.int64).to(self.device)
+        packed_i = ops.upload(ints, torch.int64, self.device)
         top_p = packed_f[1] if any(p < 1.0 for p in top_ps) else None
         return lambda logits, step, out: ops.sample(logits, packed_f[0], top_p, packed_i[0], packed_i[1 + step],
                                                     out=out)

@@ -337,3 +337,95 @@ def test_decode_runs_between_host_checks():
     t.cache.advance("r", 28)
     t.commit(plan, [5])
     assert t.plan_decode_run(10) == 3
+
+
+# ----------------------------------------------- the host one step behind
+def drive_one_step_behind(sched, max_steps=10_000):
+    """As :func:`drive`, but a step's tokens reach the scheduler only after the next step is planned
+    and committed (the engine's overlapped steps): ``commit`` without tokens, ``resolve`` a step later."""
+    from fastgen_amd.engine.scheduler import PENDING
+
+    in_flight = None
+    for _ in range(max_steps):
+        if not sched.has_work() and in_flight is None:
+            break
+        plan = sched.plan()
+        sched.finished.clear()
+        if plan:
+            assert sum(e.n for e in plan) <= sched.max_step_tokens
+            for e in plan:
+                assert e.start == e.request.n_fed == sched.cache.length(e.request.rid)
+                toks = e.request.tokens_from(e.start, e.n)
+                assert PENDING not in toks or (e.n == 1 and in_flight is not None and
+                                               any(p.request is e.request and p.wants_logits for p in in_flight[0]))
+                sched.cache.advance(e.request.rid, e.n)
+            sched.cache.check()
+            tokens = [fake_token(e.request, e.start + e.n) for e in plan if e.wants_logits]
+            sched.commit(plan)  # the tokens are "still on the device"
+        if in_flight is not None:
+            sched.resolve(*in_flight)
+            in_flight = None
+        if plan:
+            in_flight = (plan, tokens)
+    else:
+        raise AssertionError("the scheduler did not finish")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_one_step_behind_gives_the_same_requests(seed):
+    """Random loads with stop ids, small budgets and few pages (preemption): every request ends with the
+    same tokens and for the same reason whether the scheduler sees a step's tokens at once or a step
+    late; nothing is left pending, no page is lost."""
+    def load():
+        rng = random.Random(100 + seed)
+        s = mk(cache_pages=rng.choice([8, 12, 40]), page=16, max_batch=rng.choice([2, 4, 8]),
+               budget=rng.choice([8, 24, 100]), max_seq=rng.choice([None, 60]))
+        reqs = []
+        for i in range(14):
+            n = rng.choice([1, 3, 20, 45, 90])
+            if s.max_seq <= n:
+                n = 3
+            r = Request(i, [rng.randrange(50) for _ in range(n)], max_new=rng.choice([1, 5, 30]))
+            if rng.random() < 0.5:  # a stop id that the stand-in model samples at some step, or never
+                r.stop_ids = (fake_token(r, n + rng.randrange(0, 12)), 2)
+            reqs.append(r)
+            s.add(r)
+        return s, reqs
+
+    s1, reqs1 = load()
+    drive(s1)
+    s2, reqs2 = load()
+    drive_one_step_behind(s2)
+    for a, b in zip(reqs1, reqs2):
+        assert b.n_pending == 0 and -1 not in b.generated
+        assert (a.generated, a.finish_reason) == (b.generated, b.finish_reason), a.rid
+    assert s2.cache.live_requests() == [] and s2.cache.free_pages() == s1.cache.free_pages()
+    s2.cache.check()
+
+
+def test_a_stop_id_seen_a_step_late_drops_the_step_after_it():
+    from fastgen_amd.engine.scheduler import PENDING
+
+    s = mk()
+    r = Request("a", [1, 2, 3], max_new=10, stop_ids=(77,), want_logprobs=True)
+    s.add(r)
+    p0 = s.plan()
+    s.cache.advance("a", 3)
+    assert s.commit(p0) == [] and r.generated == [PENDING] and r.n_pending == 1
+    p1 = s.plan()  # planned from the count alone: one token, value unknown
+    assert [(e.start, e.n, e.wants_logits) for e in p1] == [(3, 1, True)] and r.tokens_from(3, 1) == [PENDING]
+    s.cache.advance("a", 1)
+    s.commit(p1)
+    assert r.generated == [PENDING, PENDING]
+    assert s.resolve(p0, [77], [-0.5]) == [r]  # the first token was a stop id
+    assert r.generated == [77] and r.logprobs == [-0.5] and r.finish_reason == "stop" and r.n_pending == 0
+    assert not s.has_work() and s.cache.live_requests() == []
+    assert s.resolve(p1, [5], [-1.0]) == [] and r.generated == [77]  # what the step after it sampled is dropped
+    # a request that its token count ended: the stop id found later is the reason
+    q = Request("b", [1], max_new=1, stop_ids=(9,))
+    s.add(q)
+    p = s.plan()
+    s.cache.advance("b", 1)
+    assert s.commit(p) == [q] and q.finish_reason == "length"
+    s.resolve(p, [9])
+    assert q.finish_reason == "stop" and q.generated == [9]
