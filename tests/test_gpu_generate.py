@@ -250,6 +250,39 @@ def test_stop_ids_and_logprobs(tiny_b):
     assert done[0].logprobs == pytest.approx(want, abs=1e-4)
 
 
+@pytest.mark.parametrize("overlap", [True, False])
+def test_single_steps_with_the_host_a_step_behind(tiny_b, overlap):
+    """More requests than places, so that steps are single steps: with the host one step behind
+    the device (a stop id is seen a step late, log-probabilities arrive a step late) and with every
+    step waited for, each request gets the tokens and log-probabilities of the plain implementation."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=1024, max_batch=2,
+                             max_step_tokens=48, overlap_steps=overlap)
+    prompts = tiny_b["prompts"][:5]
+    want_tokens, params = [], []
+    for i, p in enumerate(prompts):
+        free = plain_greedy(tiny_b["weights"], TINY_B, p, 9)
+        stop = (free[3 + i % 3],) if i % 2 == 0 else ()
+        if stop:
+            free = free[: free.index(stop[0]) + 1]
+        want_tokens.append(free)
+        params.append(SamplingParams(max_new_tokens=9, stop_ids=stop, logprobs=True))
+    rids = [eng.add_request(p, sp) for p, sp in zip(prompts, params)]
+    done = {}
+    while eng.has_work():
+        for r in eng.step():
+            assert r.rid not in done and r.n_pending == 0
+            done[r.rid] = r
+    assert eng.runner.cache.live_requests() == []
+    for rid, p, want in zip(rids, prompts, want_tokens):
+        r = done[rid]
+        assert r.generated == want and r.finish_reason == ("stop" if len(want) < 9 or want[-1] in r.stop_ids else "length")
+        lp = torch.log_softmax(plain_forward(tiny_b["weights"], TINY_B, p + r.generated), -1)
+        assert r.logprobs == pytest.approx([float(lp[len(p) - 1 + i, t]) for i, t in enumerate(r.generated)], abs=1e-4)
+
+
 def test_reference_style_interface(tiny_b):
     from fastgen_amd.generate import Fastgen, GenArgs, Packet
 
