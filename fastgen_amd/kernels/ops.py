@@ -52,7 +52,13 @@ def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)  # the stream's handle without a Stream object
+
+
 def _stream(t: torch.Tensor) -> ctypes.c_void_p:
+    """The device's current stream (a few hundred launches a step ask for it)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
