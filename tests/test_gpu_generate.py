@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from helpers import save_model_folder
-from plain_llama import TINY_A, TINY_B, plain_forward, plain_greedy, plain_random_weights
+from plain_llama import TINY_A, TINY_B, TINY_C, plain_forward, plain_greedy, plain_random_weights
 
 pytestmark = pytest.mark.gpu
 REPO = Path(__file__).resolve().parent.parent
@@ -281,6 +281,53 @@ def test_single_steps_with_the_host_a_step_behind(tiny_b, overlap):
         assert r.generated == want and r.finish_reason == ("stop" if len(want) < 9 or want[-1] in r.stop_ids else "length")
         lp = torch.log_softmax(plain_forward(tiny_b["weights"], TINY_B, p + r.generated), -1)
         assert r.logprobs == pytest.approx([float(lp[len(p) - 1 + i, t]) for i, t in enumerate(r.generated)], abs=1e-4)
+
+
+@pytest.mark.parametrize("dtype,stops", [(torch.bfloat16, False), (torch.float32, True)])
+def test_overlap_and_graphs_do_not_change_a_token(dtype, stops, monkeypatch):
+    """A load of 120 requests (prompts of 1..700 tokens, greedy and sampled, log-probabilities, few
+    places so that requests wait and steps are single steps) gives every request the same tokens,
+    end and log-probabilities with steps overlapped or waited for and decode steps captured or
+    not.  In float32, where no result depends on the batch, also with stop ids (which an overlapped
+    step sees a step late, so that later batches differ); in bfloat16 without them."""
+    import random
+
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    cfg = dict(TINY_C, hidden_size=512, intermediate_size=1376, num_attention_heads=8, num_key_value_heads=2,
+               num_hidden_layers=2, vocab_size=2051, max_position_embeddings=1024)
+    rng = random.Random(5)
+    n = 120
+    plens = [rng.choice([1, 2, 7, 63, 64, 65, 200, 700]) + rng.randint(0, 30) for _ in range(n)]
+    olens = [rng.choice([1, 2, 5, 40, 90]) for _ in range(n)]
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, cfg["vocab_size"], (k,), generator=g).tolist() for k in plens]
+
+    def run(overlap, graphs):
+        monkeypatch.setenv("FG_NO_GRAPHS", "0" if graphs else "1")
+        eng = Engine.from_config(cfg, seed=3, dtype=dtype, page_size=32, max_tokens=20 * 1100, max_batch=20,
+                                 max_step_tokens=300, overlap_steps=overlap, sync_freq=6)
+        assert eng.runner.use_graphs == graphs
+        for i, (p, o) in enumerate(zip(prompts, olens)):
+            eng.add_request(p, SamplingParams(
+                temperature=0.0 if i % 3 else 0.8, top_p=0.9, seed=1000 + i, max_new_tokens=o,
+                stop_ids=(17, 1042, 2000, 5, 900) if stops and i % 2 == 0 else (), logprobs=(i % 5 == 0)), rid=i)
+        out = {}
+        while eng.has_work():
+            for r in eng.step():
+                assert r.rid not in out and r.n_pending == 0
+                out[r.rid] = (list(r.generated), r.finish_reason, list(r.logprobs))
+        assert eng.runner.cache.live_requests() == []
+        eng.runner.cache.check()
+        return out
+
+    base = run(False, True)
+    assert len(base) == n and all(len(base[i][0]) <= olens[i] for i in base)
+    if stops:
+        assert any(v[1] == "stop" for v in base.values())
+    for overlap, graphs in ((True, True), (True, False), (False, False)):
+        assert run(overlap, graphs) == base, (overlap, graphs)
 
 
 def test_reference_style_interface(tiny_b):
