@@ -621,15 +621,17 @@ extern "C" int fg_attn_plan(const int* items, int n_items, int window, int max_c
 }
 
 // plan: what fg_attn_plan made of the items, with the same n_items, max_chunks and window.
+// max_rows: no item has more rows (tokens x heads of a kv head's group) than this, at most 16.
 // part_o: fp32 [max_chunks * n_kv * 16 * HD], part_ml: the same rows x 2.
 extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                              const void* v_pages, const int* block_table, int bt_stride, const int* plan,
-                             int n_items, int max_chunks, float* part_o, float* part_ml, int n_heads, int n_kv,
-                             int hd, int page_size, float scale, int window, hipStream_t stream) {
+                             int n_items, int max_chunks, int max_rows, float* part_o, float* part_ml,
+                             int n_heads, int n_kv, int hd, int page_size, float scale, int window,
+                             hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
   if (hd != HD || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > 16 || page_size < 8 || page_size % 8 ||
       !(scale > 0.f) || max_chunks < 2 * n_items || max_chunks > 65535 || n_kv > 65535 || window < 0 ||
-      q_stride % 8 || out_stride % 4 || !plan || !part_o || !part_ml)
+      q_stride % 8 || out_stride % 4 || !plan || !part_o || !part_ml || max_rows < 1 || max_rows > 16)
     return FG_ERR_ARG;
 #define LAUNCH(PERM)                                                                                           \
   attn_split_kernel<PERM><<<dim3(n_kv, max_chunks), 256, 0, stream>>>(                                         \
@@ -638,8 +640,8 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
       page_shift_of(page_size), scale, window)
   if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
 #undef LAUNCH
-  if ((long long)max_chunks * n_kv * 16 <= COMBINE_ROWS_MAX_GROUPS)
-    attn_combine_rows_kernel<<<dim3(16, n_kv, max_chunks), HD < 64 ? 64 : HD, 0, stream>>>(
+  if ((long long)max_chunks * n_kv * max_rows <= COMBINE_ROWS_MAX_GROUPS)
+    attn_combine_rows_kernel<<<dim3(max_rows, n_kv, max_chunks), HD < 64 ? 64 : HD, 0, stream>>>(
         part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
   else
     attn_combine_kernel<<<dim3(n_kv, max_chunks), 256, 0, stream>>>(

@@ -336,12 +336,13 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan: Optional[torch.Tensor] = None, max_chunks: Optional[int] = None,
-                         min_tiles: int = 4) -> torch.Tensor:
+                         min_tiles: int = 4, max_rows: int = 16) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
     device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
     every query token of the step must be covered by exactly one item.
     ``plan``: :func:`attention_plan` of the small items with this ``max_chunks``
-    and ``window`` (made here if not given)."""
+    and ``window`` (made here if not given).  ``max_rows``: no small item has
+    more rows (tokens times query heads per kv head) than this."""
     _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
@@ -360,7 +361,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     lib = _lib.load(f"attention_mfma@{hd}")
     G = n_heads // n_kv
     if small_items is not None and small_items.numel():
-        _need(G <= 16, "the split kernel takes at most 16 query heads per kv head")
+        _need(G <= 16 and 1 <= max_rows <= 16, "the split kernel takes at most 16 rows an item")
         _i32(small_items, "small_items")
         _need(small_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
         n = small_items.numel() // 4
@@ -375,7 +376,7 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
         part_ml = torch.empty((max_chunks * n_kv * 16, 2), dtype=torch.float32, device=q.device)
         st = lib.fg_attn_split(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            block_table.stride(0), _ptr(plan), n, max_chunks, _ptr(part_o), _ptr(part_ml), n_heads, n_kv, hd,
+            block_table.stride(0), _ptr(plan), n, max_chunks, max_rows, _ptr(part_o), _ptr(part_ml), n_heads, n_kv, hd,
             page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
         _check(st, "attn_split")
     if big_items is not None and big_items.numel():
@@ -425,8 +426,10 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
         split_plan = ctx.scratch.get(key)
         if split_plan is None:
             split_plan = ctx.scratch[key] = attention_plan(small_d, n_small, chunks, hd, window, _SPLIT_MIN_TILES)
+    # rows of the largest small item: one token a sequence in a decode step (also a captured one)
+    rows = G * int(ctx.q_lens.max()) if big_d is None else 16
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
-                                window, split_plan, chunks)
+                                window, split_plan, chunks, max_rows=min(16, rows))
 
 
 # ----------------------------------------------------------------------- gemm
