@@ -55,10 +55,10 @@ LLAMA_70B = dict(
 SHAPES = {"8b": ("llama-3.1-8b-shape-random", LLAMA_8B), "70b": ("llama-3.1-70b-shape-random", LLAMA_70B)}
 
 
-def serve_workload(n_requests: int = 256) -> int:
+def serve_workload(n_requests: int = 256, step_budget: int = 2048) -> int:
     """Continuous batching at the Llama 3.2 3B shape (random bfloat16 weights): ``n_requests`` requests
     arrive at once, prompts of 128..4096 uniform random ids, 32..512 greedy tokens each, at most 256 live,
-    a budget of 2,048 tokens a step (prompt portions beside decoded tokens).  One JSON line: generated
+    a budget of ``step_budget`` tokens a step (prompt portions beside decoded tokens).  One JSON line: generated
     tokens a second over the whole run, prompt processing included."""
     import random
 
@@ -72,7 +72,7 @@ def serve_workload(n_requests: int = 256) -> int:
     olens = [rng.randint(32, 512) for _ in range(n_requests)]
     max_batch = min(256, n_requests)
     engine = Engine.from_config(LLAMA_3B, seed=3, dtype=torch.bfloat16, page_size=PAGE, max_tokens=max_batch * 4672,
-                                max_batch=max_batch, max_step_tokens=2048)
+                                max_batch=max_batch, max_step_tokens=step_budget)
     g = torch.Generator().manual_seed(0)
     prompts = [torch.randint(0, LLAMA_3B["vocab_size"], (n,), generator=g).tolist() for n in plens]
     torch.cuda.synchronize()
@@ -91,7 +91,7 @@ def serve_workload(n_requests: int = 256) -> int:
         "metric": "generated tok/s, continuous batching", "value": round(sum(olens) / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"model": "llama-3.2-3b-shape-random", "requests": n_requests, "prompt_tokens": sum(plens),
-                   "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": 2048, "page_size": PAGE,
+                   "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": step_budget, "page_size": PAGE,
                    "engine_steps": engine.n_steps, "preemptions": engine.scheduler.n_preemptions},
     }), flush=True)
     return 0
@@ -144,12 +144,13 @@ def main() -> int:
     ap.add_argument("--workload", choices=["decode", "serve", "readme"], default="decode",
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
                          "readme: the load of the reference's README")
+    ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported", flush=True)
         return 2
     if a.workload == "serve":
-        return serve_workload()
+        return serve_workload(step_budget=a.step_budget)
     if a.workload == "readme":
         return readme_workload()
 
