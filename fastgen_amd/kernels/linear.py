@@ -56,10 +56,11 @@ def wide_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[0] <= WIDE_ROWS and _aligned(x, w)
 
 
-def k_splits_for(n_out: int, k: int) -> int:
-    """Splits of the k range that give the wide kernel about two workgroups per CU."""
+def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
+    """Splits of the k range that give the wide kernel about two workgroups per CU; with many rows
+    a split keeps at least 1,024 of k (the partial sums it writes grow with the rows)."""
     blocks = -(-n_out // 64)
-    return max(1, min(8, 512 // blocks, k // 512))
+    return max(1, min(8, 512 // blocks, k // (1024 if rows > 48 else 512)))
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -77,7 +78,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
     if partials_ok and x.shape[0] > 2 and wide_ok(x, w) and w.shape[0] <= 8192:
-        splits = k_splits_for(w.shape[0], w.shape[1])
+        splits = k_splits_for(w.shape[0], w.shape[1], x.shape[0])
         if splits > 1:
             return ops.gemm_skinny(x, w, k_splits=splits, wide=True)
     if skinny_ok(x, w):
