@@ -416,3 +416,26 @@ def test_smoke_entry():
     import __graft_entry__
 
     __graft_entry__.smoke()
+
+
+def test_bench_line():
+    """bench.py with one of the 32 layers and a few steps: one JSON line with the fields of its
+    contract (value = decoded tokens a second, prefill, roofline, a flat config that names both
+    layer counts)."""
+    import json
+
+    bench = Path(__file__).resolve().parent.parent / "bench.py"
+    r = subprocess.run([sys.executable, str(bench), "--layers", "1", "--steps", "3", "--warmup", "1", "--no-points"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+    assert len(lines) == 1
+    j = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline"):
+        assert key in j, key
+    assert j["n_gpus"] == 1 and j["steps"] == 3 and j["warmup"] == 1 and j["dtype"] == "bf16" and j["value"] > 0
+    assert j["config"]["layers"] == 1 and j["config"]["layers_full"] == 32 and len(j["config"]) <= 20
+    assert all(not isinstance(v, (dict, list)) for v in j["config"].values())
+    assert set(j["prefill"]) == {"value", "tokens", "ms", "frac"} and j["prefill"]["tokens"] == 2048
+    assert j["roofline"]["bound"] == "hbm" and j["roofline"]["peak"] == 8000.0 and 0 < j["roofline"]["frac"] < 1
