@@ -54,6 +54,9 @@ class Request:
     n_pending: int = 0  # PENDING places in ``generated``
     preemptions: int = 0
     finish_reason: Optional[str] = None
+    # a request whose prompt and ``max_new`` tokens can never be held by the cache at once is
+    # refused when it is added, unless it agrees to end early (reason ``max_seq``)
+    truncate: bool = False
 
     def all_tokens(self) -> List[int]:
         return self.prompt + self.generated
@@ -94,12 +97,14 @@ class Scheduler:
         self.max_batch = min(max_batch, cache.n_slots)
         self.max_step_tokens = max_step_tokens
         pool_tokens = min(cache.n_pages) * cache.page_size if cache.n_groups else 1 << 62
+        self.pool_tokens = pool_tokens
         self.max_seq = min(max_seq or pool_tokens, pool_tokens)
         self._admit = on_admit or cache.admit
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []  # in order of admission
         self.finished: List[Request] = []
         self.n_preemptions = 0
+        self._served_last: Optional[Request] = None  # the last request that step A gave a token
 
     # ------------------------------------------------------------- intake
     def add(self, req: Request) -> None:
@@ -112,6 +117,12 @@ class Scheduler:
             )
         if req.max_new < 1:
             raise ValueError(f"request {req.rid!r}: max_new must be at least 1")
+        # the reference clamps silently: maxlen = min(len + max_gen, max_seq), fastgen/generate.py:95-113
+        if len(req.prompt) + req.max_new > self.pool_tokens and not req.truncate:
+            raise ValueError(
+                f"request {req.rid!r}: a prompt of {len(req.prompt)} tokens and {req.max_new} new ones can never"
+                f" fit: the cache holds {self.pool_tokens} tokens (ask for fewer, or let it be cut short: truncate)"
+            )
         self.waiting.append(req)
 
     def has_work(self) -> bool:
@@ -143,6 +154,10 @@ class Scheduler:
             self.cache.release(req.rid)
         if req in self.running:
             self.running.remove(req)
+        # a request preempted with a sample still on the device waits for re-admission; when that
+        # sample turns out to be a stop id it must not be admitted again
+        if any(r is req for r in self.waiting):
+            self.waiting = deque(r for r in self.waiting if r is not req)
         self.finished.append(req)
 
     def _fits(self, req: Request, n: int) -> int:
@@ -159,8 +174,13 @@ class Scheduler:
         budget = self.max_step_tokens
         gone = set()  # ids of requests preempted or ended while planning
         # A. one token for every decoding request, oldest first; make room by
-        #    preempting the youngest
-        for req in list(self.running):
+        #    preempting the youngest.  A budget smaller than the number of decoding
+        #    requests goes round: the walk starts behind the request served last.
+        walk = list(self.running)
+        if budget < len(walk) and any(r is self._served_last for r in walk):
+            at = next(i for i, r in enumerate(walk) if r is self._served_last) + 1
+            walk = walk[at:] + walk[:at]
+        for req in walk:
             if budget == 0:
                 break
             if id(req) in gone or req.remaining() != 1:
@@ -181,6 +201,7 @@ class Scheduler:
                 continue
             self.cache.reserve(req.rid, 1)
             entries.append(PlannedEntry(req, req.n_fed, 1, True))
+            self._served_last = req
             budget -= 1
         budget = self.max_step_tokens - sum(e.n for e in entries)
         planned = {id(e.request) for e in entries}

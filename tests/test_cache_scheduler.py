@@ -258,7 +258,7 @@ def test_out_of_pages_preempts_the_youngest_and_recomputes():
 
 def test_alone_and_out_of_pages_ends_with_cache_full():
     s = mk(cache_pages=2, max_batch=1, budget=64, max_seq=1000)
-    r = Request("a", [1] * 20, max_new=100)
+    r = Request("a", [1] * 20, max_new=100, truncate=True)
     s.add(r)
     drive(s)
     assert r.finish_reason in ("cache_full", "max_seq") and r.n_known() <= 32
@@ -321,7 +321,7 @@ def test_decode_runs_between_host_checks():
     # pages: a run must fit for all requests at once
     for pages, want in ((4, 10), (3, 0)):
         t = mk(cache_pages=pages, max_batch=2, budget=64)
-        rs = [Request(i, [1] * 15, max_new=40) for i in range(2)]
+        rs = [Request(i, [1] * 15, max_new=40, truncate=True) for i in range(2)]
         for r in rs:
             t.add(r)
         plan = t.plan()
@@ -331,7 +331,7 @@ def test_decode_runs_between_host_checks():
         assert t.plan_decode_run(10) == want
     # the cap of one request's length (here the pool itself) bounds a run
     t = mk(cache_pages=2, max_batch=1, budget=64)
-    r = Request("r", [1] * 28, max_new=50)
+    r = Request("r", [1] * 28, max_new=50, truncate=True)
     t.add(r)
     plan = t.plan()
     t.cache.advance("r", 28)
@@ -346,14 +346,17 @@ def drive_one_step_behind(sched, max_steps=10_000):
     from fastgen_amd.engine.scheduler import PENDING
 
     in_flight = None
+    reported = []
     for _ in range(max_steps):
+        reported += [r.rid for r in sched.finished]
+        sched.finished.clear()
         if not sched.has_work() and in_flight is None:
             break
         plan = sched.plan()
-        sched.finished.clear()
         if plan:
             assert sum(e.n for e in plan) <= sched.max_step_tokens
             for e in plan:
+                assert e.request.finish_reason is None, "a request that has ended runs again"
                 assert e.start == e.request.n_fed == sched.cache.length(e.request.rid)
                 toks = e.request.tokens_from(e.start, e.n)
                 assert PENDING not in toks or (e.n == 1 and in_flight is not None and
@@ -369,23 +372,26 @@ def drive_one_step_behind(sched, max_steps=10_000):
             in_flight = (plan, tokens)
     else:
         raise AssertionError("the scheduler did not finish")
+    return reported
 
 
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(16))
 def test_one_step_behind_gives_the_same_requests(seed):
     """Random loads with stop ids, small budgets and few pages (preemption): every request ends with the
     same tokens and for the same reason whether the scheduler sees a step's tokens at once or a step
     late; nothing is left pending, no page is lost."""
     def load():
         rng = random.Random(100 + seed)
-        s = mk(cache_pages=rng.choice([8, 12, 40]), page=16, max_batch=rng.choice([2, 4, 8]),
+        # odd seeds: pools so tight that decoding requests are preempted with a sample still pending
+        pages = rng.choice([8, 12, 40]) if seed % 2 == 0 else rng.choice([7, 8, 9])
+        s = mk(cache_pages=pages, page=16, max_batch=rng.choice([2, 4, 8]),
                budget=rng.choice([8, 24, 100]), max_seq=rng.choice([None, 60]))
         reqs = []
         for i in range(14):
-            n = rng.choice([1, 3, 20, 45, 90])
+            n = rng.choice([1, 3, 20, 45, 90]) if seed % 2 == 0 else rng.choice([7, 15, 30, 31, 47])
             if s.max_seq <= n:
                 n = 3
-            r = Request(i, [rng.randrange(50) for _ in range(n)], max_new=rng.choice([1, 5, 30]))
+            r = Request(i, [rng.randrange(50) for _ in range(n)], max_new=rng.choice([1, 5, 30]), truncate=True)
             if rng.random() < 0.5:  # a stop id that the stand-in model samples at some step, or never
                 r.stop_ids = (fake_token(r, n + rng.randrange(0, 12)), 2)
             reqs.append(r)
@@ -395,7 +401,8 @@ def test_one_step_behind_gives_the_same_requests(seed):
     s1, reqs1 = load()
     drive(s1)
     s2, reqs2 = load()
-    drive_one_step_behind(s2)
+    reported = drive_one_step_behind(s2)
+    assert sorted(reported) == list(range(14))  # every request is reported as ended exactly once
     for a, b in zip(reqs1, reqs2):
         assert b.n_pending == 0 and -1 not in b.generated
         assert (a.generated, a.finish_reason) == (b.generated, b.finish_reason), a.rid
@@ -429,3 +436,72 @@ def test_a_stop_id_seen_a_step_late_drops_the_step_after_it():
     assert s.commit(p) == [q] and q.finish_reason == "length"
     s.resolve(p, [9])
     assert q.finish_reason == "stop" and q.generated == [9]
+
+
+def test_a_late_stop_id_of_a_preempted_request_ends_it_once():
+    """A decoding request is preempted while its last sample is still on the device; the sample
+    turns out to be a stop id.  The request ends there: it is in neither line, is reported once,
+    and is never admitted again."""
+    s = mk(cache_pages=2, page=8, max_batch=2, budget=64)
+    a, b = Request("a", [1] * 7, max_new=8, stop_ids=(99,)), Request("b", [2] * 7, max_new=8, stop_ids=(99,))
+    s.add(a), s.add(b)
+    p0 = s.plan()
+    assert [(e.request.rid, e.n) for e in p0] == [("a", 7), ("b", 7)]
+    for e in p0:
+        s.cache.advance(e.request.rid, e.n)
+    assert s.commit(p0) == []  # both samples pending
+    p1 = s.plan()  # a and b decode: the 8th token still fits each one's page
+    for e in p1:
+        s.cache.advance(e.request.rid, e.n)
+    s.commit(p1)
+    s.resolve(p0, [7, 6])
+    p2 = s.plan()  # the 9th token of a needs a page: b, the youngest, gives way with a sample pending
+    assert [e.request.rid for e in p2] == ["a"] and b.preemptions == 1 and b.n_pending == 1
+    assert any(r is b for r in s.waiting)
+    s.cache.advance("a", 1)
+    s.commit(p2)
+    late = s.resolve(p1, [8, 99])  # b's pending token is a stop id
+    assert late == [b] and b.finish_reason == "stop" and b.generated == [6, 99]
+    assert not any(r is b for r in s.waiting) and not any(r is b for r in s.running)
+    assert [r.rid for r in s.finished].count("b") == 1
+    s.finished.clear()
+    s.resolve(p2, [9])
+    reported = drive_one_step_behind(s)
+    assert "b" not in reported and b.generated == [6, 99] and a.finish_reason == "length"
+    assert s.cache.live_requests() == [] and s.cache.free_pages() == 2
+
+
+def test_a_request_that_can_never_fit_is_refused_unless_it_agrees_to_be_cut():
+    s = mk(cache_pages=4, page=16, max_batch=2, budget=64)  # 64 tokens of cache
+    with pytest.raises(ValueError, match="can never fit.*holds 64 tokens"):
+        s.add(Request("a", [1] * 40, max_new=25))
+    assert not s.has_work()
+    s.add(Request("b", [1] * 40, max_new=24))  # 64 exactly: fits
+    r = Request("c", [1] * 40, max_new=100, truncate=True)
+    s.add(r)
+    drive(s)
+    assert r.finish_reason == "max_seq" and r.n_known() == 64
+
+
+def test_a_budget_smaller_than_the_decoding_requests_goes_round():
+    """max_step_tokens < live decoders: every request advances, none is left out of every step."""
+    s = mk(cache_pages=64, page=16, max_batch=5, budget=5)
+    reqs = [Request(i, [i + 1], max_new=12) for i in range(5)]
+    for r in reqs:
+        s.add(r)
+    plan = s.plan()  # all five prompts
+    for e in plan:
+        s.cache.advance(e.request.rid, e.n)
+    s.commit(plan, [5] * 5)
+    s.max_step_tokens = 2
+    served = {r.rid: 0 for r in reqs}
+    for _ in range(10):
+        plan = s.plan()
+        assert sum(e.n for e in plan) <= 2
+        for e in plan:
+            served[e.request.rid] += 1
+            s.cache.advance(e.request.rid, e.n)
+        s.commit(plan, [5] * sum(e.wants_logits for e in plan))
+    assert max(served.values()) - min(served.values()) <= 1, served
+    drive(s)
+    assert all(len(r.generated) == 12 for r in reqs)
