@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
     python bench.py --workload serve        # continuous batching, see serve_workload()
     python bench.py --workload readme       # the load of the reference's README, see readme_workload()
+    python bench.py --workload readme --shape 70b   # the same load at the 70B sizes, cache = the memory left
 
 The model has the layer sizes of Llama 3.1 8B (32 layers, hidden 4096, 32
 heads, 8 kv heads, head size 128, feed-forward 14336, vocabulary 128256,
@@ -52,10 +53,11 @@ LLAMA_70B = dict(
                       original_max_position_embeddings=8192),
     tie_word_embeddings=False, max_position_embeddings=131072,
 )
-SHAPES = {"8b": ("llama-3.1-8b-shape-random", LLAMA_8B), "70b": ("llama-3.1-70b-shape-random", LLAMA_70B)}
+SHAPES = {"3b": ("llama-3.2-3b-shape-random", LLAMA_3B), "8b": ("llama-3.1-8b-shape-random", LLAMA_8B),
+          "70b": ("llama-3.1-70b-shape-random", LLAMA_70B)}
 
 
-def serve_workload(n_requests: int = 256, step_budget: int = 2048) -> int:
+def serve_workload(n_requests: int = 256, step_budget: int = 2048, shape: str = "3b") -> int:
     """Continuous batching at the Llama 3.2 3B shape (random bfloat16 weights): ``n_requests`` requests
     arrive at once, prompts of 128..4096 uniform random ids, 32..512 greedy tokens each, at most 256 live,
     a budget of ``step_budget`` tokens a step (prompt portions beside decoded tokens).  One JSON line: generated
@@ -71,10 +73,11 @@ def serve_workload(n_requests: int = 256, step_budget: int = 2048) -> int:
     plens = [rng.randint(128, 4096) for _ in range(n_requests)]
     olens = [rng.randint(32, 512) for _ in range(n_requests)]
     max_batch = min(256, n_requests)
-    engine = Engine.from_config(LLAMA_3B, seed=3, dtype=torch.bfloat16, page_size=PAGE, max_tokens=max_batch * 4672,
+    model_name, cfg = SHAPES[shape]
+    engine = Engine.from_config(cfg, seed=3, dtype=torch.bfloat16, page_size=PAGE, max_tokens=max_batch * 4672,
                                 max_batch=max_batch, max_step_tokens=step_budget)
     g = torch.Generator().manual_seed(0)
-    prompts = [torch.randint(0, LLAMA_3B["vocab_size"], (n,), generator=g).tolist() for n in plens]
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in plens]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for p, o in zip(prompts, olens):
@@ -90,42 +93,68 @@ def serve_workload(n_requests: int = 256, step_budget: int = 2048) -> int:
     print(json.dumps({
         "metric": "generated tok/s, continuous batching", "value": round(sum(olens) / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
-        "config": {"model": "llama-3.2-3b-shape-random", "requests": n_requests, "prompt_tokens": sum(plens),
+        "config": {"model": model_name, "requests": n_requests, "prompt_tokens": sum(plens),
                    "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": step_budget, "page_size": PAGE,
                    "engine_steps": engine.n_steps, "preemptions": engine.scheduler.n_preemptions},
     }), flush=True)
     return 0
 
 
-def readme_workload() -> int:
-    """The load behind the numbers of the reference's README (``README.md:22-28``: 512 prompts of 1,024
-    tokens, 128 decode steps each, generated tokens over the wall-clock time of the whole batch), at the
-    Llama 3.1 8B shape with random bfloat16 weights and uniform random ids.  The reference publishes 3,430
-    tok/s for Mistral 7B on one H100 through its server: another model and other hardware, so the ratio in
+def readme_workload(shape: str = "8b") -> int:
+    """The load behind the numbers of the reference's README (``README.md:22-28``, ``scripts/bench.py:104-106``:
+    512 prompts of 1,024 tokens, 128 decode steps each, generated tokens over the wall-clock time of the whole
+    batch), with random bfloat16 weights and uniform random ids, at the Llama 3.1 8B shape or, ``--shape 70b``, at
+    the 70B shape (141 GB of weights).  The cache is what the GPU has free once the weights are in place
+    (``fastgen/utils/tune.py:68-84`` sizes it from a budget): at 8B it holds all 512 requests, at 70B it does not
+    and requests are preempted and recomputed.  The reference publishes 3,430 tok/s for Mistral 7B on one H100 and
+    2,260 tok/s for Llama 70B on eight, through its server: other models and other hardware, so the ratio in
     ``vs_published`` is context, not a like-for-like comparison."""
     import torch
 
-    from fastgen_amd.engine import Engine
+    from fastgen_amd.engine import Engine, Model
     from fastgen_amd.sampling import SamplingParams
 
     n, p_len, n_gen, max_batch = 512, 1024, 128, 512
-    engine = Engine.from_config(LLAMA_8B, seed=2, dtype=torch.bfloat16, page_size=PAGE,
-                                max_tokens=max_batch * (p_len + n_gen + PAGE), max_batch=max_batch, max_step_tokens=8192)
-    g = torch.Generator().manual_seed(0)
-    prompts = [torch.randint(0, LLAMA_8B["vocab_size"], (p_len,), generator=g).tolist() for _ in range(n)]
-    torch.cuda.synchronize()
+    model_name, cfg = SHAPES[shape]
+    published = {"8b": (3430.0, "3430 tok/s, Mistral 7B, 1x H100 (reference README)"),
+                 "70b": (2260.0, "2260 tok/s, Llama 70B, 8x H100 (reference README)")}.get(shape)
     t0 = time.perf_counter()
-    out = engine.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=n_gen))
+    model = Model.random(cfg, 4 if shape == "70b" else 2, torch.bfloat16, "cuda:0")
+    torch.cuda.synchronize()
+    print(f"[bench] model built in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)
+    # no request is longer than prompt + generated: the cache never needs more than that for each
+    engine = Engine(model, page_size=PAGE, max_tokens=None, max_batch=max_batch, max_step_tokens=8192,
+                    max_seq=-(-(p_len + n_gen) // PAGE) * PAGE)
+    pool = engine.scheduler.pool_tokens
+    print(f"[bench] cache of {pool} tokens ({pool * engine.runner.storage.bytes_per_token() / 1e9:.1f} GB)",
+          file=sys.stderr, flush=True)
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, cfg["vocab_size"], (p_len,), generator=g).tolist() for _ in range(n)]
+    params = SamplingParams(temperature=0.0, max_new_tokens=n_gen)
+    torch.cuda.synchronize()
+    t0 = last = time.perf_counter()
+    for p in prompts:
+        engine.add_request(p, params)
+    generated = n_done = 0
+    while engine.has_work():
+        for r in engine.step():
+            generated += len(r.generated)
+            n_done += 1
+        if time.perf_counter() - last > 20:
+            last = time.perf_counter()
+            print(f"[bench] {n_done}/{n} requests done, {engine.scheduler.n_preemptions} preemptions",
+                  file=sys.stderr, flush=True)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    generated = sum(len(o) for o in out)
     print(json.dumps({
         "metric": "generated tok/s, 512 prompts x 1024 tokens, 128 decode steps", "value": round(generated / dt, 1),
         "unit": "tokens/s", "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16",
-        "data": "synthetic", "vs_published": round(generated / dt / 3430.0, 3),
-        "config": {"model": "llama-3.1-8b-shape-random", "requests": n, "prompt_len": p_len, "generated": n_gen,
+        "data": "synthetic", "vs_published": round(generated / dt / published[0], 3) if published else None,
+        "config": {"model": model_name, "requests": n, "prompt_len": p_len, "generated": n_gen,
                    "max_batch": max_batch, "step_budget": 8192, "page_size": PAGE, "engine_steps": engine.n_steps,
-                   "published": "3430 tok/s, Mistral 7B, 1x H100 (reference README)"},
+                   "cache_tokens": pool, "cache": "free memory after the weights",
+                   "preemptions": engine.scheduler.n_preemptions,
+                   "published": published[1] if published else None},
     }), flush=True)
     return 0
 
@@ -137,8 +166,12 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (both numbers are reported)")
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
-                    help="layer sizes: Llama 3.1 8B (default, the benchmark's configuration) or 70B (141 GB of weights)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default=None,
+                    help="layer sizes: Llama 3.1 8B (the benchmark's configuration; default but for serve), 70B"
+                         " (141 GB of weights) or Llama 3.2 3B (the default of serve)")
+    ap.add_argument("--context", type=int, default=None,
+                    help="cached tokens of each request when the timed decode steps begin (default: the prompt's"
+                         " 2,048); more are fed untimed, in portions")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--workload", choices=["decode", "serve", "readme"], default="decode",
@@ -150,9 +183,10 @@ def main() -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported", flush=True)
         return 2
     if a.workload == "serve":
-        return serve_workload(step_budget=a.step_budget)
+        return serve_workload(step_budget=a.step_budget, shape=a.shape or "3b")
     if a.workload == "readme":
-        return readme_workload()
+        return readme_workload(a.shape or "8b")
+    a.shape = a.shape or "8b"
 
     import torch
 
@@ -166,9 +200,13 @@ def main() -> int:
     batches = sorted({a.batch} | (set() if a.no_points else {1, 64}))
     max_b = max(batches)
     t0 = time.time()
+    # the cache holds CONTEXT_LEN tokens for every request of the largest batch (68.7 GB at batch 64 of the 8B
+    # shape in bfloat16); with --context beyond it, that many
+    ctx_len = a.context or PROMPT_LEN
+    capacity = max(CONTEXT_LEN, -(-(ctx_len + a.warmup + a.steps + 64) // PAGE) * PAGE)
     engine = Engine.from_config(cfg, seed=2, dtype=dtype, page_size=PAGE,
-                                max_tokens=max_b * (PROMPT_LEN + 512), max_batch=max_b,
-                                max_step_tokens=PROMPT_LEN)
+                                max_tokens=max_b * capacity, max_batch=max_b,
+                                max_step_tokens=PROMPT_LEN, max_seq=capacity)
     torch.cuda.synchronize()
     print(f"[bench] model built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     model = engine.model
@@ -185,19 +223,21 @@ def main() -> int:
         return torch.randint(0, V, (n,), generator=g).tolist()
 
     # ------------------------------------------------------------ prefill
-    pre = engine.time_prefill(prompt(PROMPT_LEN), repeats=3)
+    times = engine.time_prefill(prompt(PROMPT_LEN), repeats=5)
+    pre = sum(times) / len(times)  # the mean of the repeats after one warm-up; the best is reported beside it
     T = PROMPT_LEN
     flops = 2 * T * L * layer_params + L * 4 * H * hd * (T * (T + 1) // 2) + 2 * D * V
     prefill = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
-               "frac": round(flops / pre / PEAK_FLOPS[a.dtype], 4)}
+               "frac": round(flops / pre / PEAK_FLOPS[a.dtype], 4), "repeats": len(times),
+               "best_ms": round(min(times) * 1e3, 3)}
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
 
     # ------------------------------------------------------------- decode
     results = {}
     for b in batches:
         steps, warm = (a.steps, a.warmup)
-        dt = engine.time_decode([prompt(PROMPT_LEN) for _ in range(b)], steps=steps, warmup=warm)
-        ctx = PROMPT_LEN + warm + steps / 2  # mean cached tokens during the timed steps
+        dt = engine.time_decode([prompt(ctx_len) for _ in range(b)], steps=steps, warmup=warm)
+        ctx = ctx_len + warm + steps / 2  # mean cached tokens during the timed steps
         nbytes = (L * layer_params + D * V) * esize + b * ctx * kv_bytes_per_token
         results[b] = dict(tok_s=b * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9)
         print(f"[bench] decode batch {b}: {results[b]}", file=sys.stderr, flush=True)
@@ -209,8 +249,8 @@ def main() -> int:
         "ms_per_step": round(r["ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
         "config": {
-            "model": model_name, "global_batch": a.batch, "seq_len": CONTEXT_LEN,
-            "prompt_len": PROMPT_LEN, "parallelism": "none", "layers": L, "layers_full": full_layers,
+            "model": model_name, "global_batch": a.batch, "seq_len": capacity, "mean_context": ctx_len + a.warmup + a.steps / 2,
+            "prompt_len": ctx_len, "cache_tokens": engine.scheduler.pool_tokens, "parallelism": "none", "layers": L, "layers_full": full_layers,
             "hidden": D, "heads": H, "kv_heads": KV, "head_dim": hd, "ffn": F, "vocab": V, "page_size": PAGE,
             "rope_theta": cfg["rope_theta"], "rope_factor": cfg["rope_scaling"]["factor"], "norm_eps": cfg["rms_norm_eps"],
         },

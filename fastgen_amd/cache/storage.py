@@ -37,6 +37,35 @@ def group_entries(needs: Sequence[Optional[PagedNeed]]) -> List[CacheGroup]:
     return [CacheGroup(n, tuple(e)) for n, e in by_need.items()]
 
 
+def bytes_per_token(groups: Sequence[CacheGroup], dtype: torch.dtype) -> int:
+    """Cache bytes one token takes over all layers of all groups."""
+    esize = torch.empty((), dtype=dtype).element_size()
+    return sum(2 * len(g.entries) * g.need.n_kv_heads * g.need.head_dim * esize for g in groups)
+
+
+def tokens_for_free_memory(groups: Sequence[CacheGroup], page_size: int, dtype: torch.dtype,
+                           device: torch.device | str, reserve_bytes: int, at_most: Optional[int] = None) -> int:
+    """The cache that the device's free memory holds beside ``reserve_bytes`` (activations of the
+    largest step, captured steps, the libraries' work space), in tokens, a whole number of pages.
+    The reference sizes its cache from a memory budget the same way (``fastgen/utils/tune.py:68-84``,
+    ``fastgen/generate.py:224-238``); here the budget is what the device reports as free now, after
+    the weights are in place.  ``at_most``: no more than this many tokens are ever needed."""
+    free, _total = torch.cuda.mem_get_info(torch.device(device))
+    # what torch's allocator holds but does not use is free for the pools as well
+    free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+    per_token = max(1, bytes_per_token(groups, dtype))
+    tokens = int((free - reserve_bytes) // per_token)
+    if at_most is not None:
+        tokens = min(tokens, at_most)
+    tokens = tokens // page_size * page_size
+    if tokens < page_size:
+        raise RuntimeError(
+            f"no room for one cache page: {free / 1e9:.2f} GB are free on {device}, {reserve_bytes / 1e9:.2f} GB"
+            f" are kept for the steps' activations, a page of {page_size} tokens takes {per_token * page_size / 1e6:.2f} MB"
+        )
+    return tokens
+
+
 class CacheStorage:
     def __init__(self, groups: Sequence[CacheGroup], pages_per_group: Sequence[int], page_size: int,
                  state_needs: Dict[int, StateNeed], n_slots: int, dtype: torch.dtype,

@@ -34,17 +34,39 @@ class _InFlight:
     copied: torch.cuda.Event
 
 
+def step_memory_estimate(model: Model, max_step_tokens: int, max_batch: int) -> int:
+    """Bytes that one step's intermediate tensors take at most: per token a few rows as wide as the
+    widest matrix product of a layer (its output, the activation made from it, the fp32 partial sums
+    of the product after it) and the fp32 residual stream; per request a row of fp32 logits, twice
+    (a captured step keeps its own).  (``fastgen/utils/tune.py:46-65`` budgets 1.2 x (4 dim + 4 ffn)
+    bytes a token for the same purpose.)"""
+    widest = model.layout.dim
+    for part in model.parts.all_parts[1:-1]:  # the layers' parts; the embedding and the head are not per token
+        for v in vars(part).values():
+            if isinstance(v, torch.Tensor) and v.dim() == 2:
+                widest = max(widest, v.shape[0])
+    return int(max_step_tokens * 12 * widest + 3 * max_batch * model.vocab_size * 4)
+
+
 class Engine:
-    def __init__(self, model: Model, page_size: int = 64, max_tokens: int = 8192, max_batch: int = 64,
+    def __init__(self, model: Model, page_size: int = 64, max_tokens: Optional[int] = 8192, max_batch: int = 64,
                  max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0,
-                 sync_freq: int = 10, overlap_steps: Optional[bool] = None) -> None:
+                 sync_freq: int = 10, overlap_steps: Optional[bool] = None,
+                 reserve_bytes: Optional[int] = None) -> None:
+        """``max_tokens``: the cache's size in tokens; None: whatever memory the device has free
+        now, the weights being in place, beside ``reserve_bytes`` (default: an estimate of what a
+        step of ``max_step_tokens`` tokens and ``max_batch`` rows of logits take, plus 2 GiB)."""
         self.model = model
-        self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch)
         cap = getattr(model.args, "max_position", 0) or None
         if max_seq is None:
             max_seq = cap
         elif cap:
             max_seq = min(max_seq, cap)
+        if reserve_bytes is None:
+            reserve_bytes = step_memory_estimate(model, max_step_tokens, max_batch) + (2 << 30)
+        at_most = max_batch * (-(-max_seq // page_size) * page_size) if max_seq else None
+        self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch,
+                                  reserve_bytes=reserve_bytes, at_most_tokens=at_most)
         self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit)
         # no request gets longer than the scheduler lets it: block tables need not be wider
         self.runner.table_width = min(self.runner.table_width, -(-self.scheduler.max_seq // page_size))
@@ -85,12 +107,13 @@ class Engine:
         if any(not 0 <= int(t) < vocab for t in prompt):
             raise ValueError(f"request {rid!r}: token id outside [0, {vocab})")
         # a request's own seed, unless it gave one: the engine's seed and its arrival number
-        seed = params.seed if params.seed else (self.seed * 1000003 + self._n_requests + 1)
+        seed = params.seed if params.seed is not None else (self.seed * 1000003 + self._n_requests + 1)
         self._n_requests += 1
         self.scheduler.add(Request(
             rid=rid, prompt=[int(t) for t in prompt], max_new=params.max_new_tokens,
             temperature=float(params.temperature), top_p=float(params.top_p), seed=seed,
-            stop_ids=tuple(params.stop_ids), want_logprobs=params.logprobs,
+            stop_ids=tuple(params.stop_ids), want_logprobs=params.logprobs, truncate=params.truncate,
+            keep_stop_token=params.keep_stop_token,
         ))
         return rid
 
@@ -186,6 +209,11 @@ class Engine:
         self.scheduler.finished.clear()
         out = [r for r in self._held if r.n_pending == 0]
         self._held = [r for r in self._held if r.n_pending]
+        for r in out:
+            if (r.finish_reason == "stop" and not r.keep_stop_token and r.generated
+                    and r.generated[-1] in r.stop_ids):
+                r.generated.pop()
+                del r.logprobs[len(r.generated):]
         return out
 
     def _decode_run(self, n_steps: int) -> List[Request]:
@@ -229,10 +257,10 @@ class Engine:
         return [out[r] for r in rids]
 
     # ------------------------------------------------------- measurement
-    def time_prefill(self, prompt: Sequence[int], repeats: int = 3) -> float:
+    def time_prefill(self, prompt: Sequence[int], repeats: int = 3) -> List[float]:
         """Seconds of one step that takes the whole prompt and returns the
-        logits of its last token (best of ``repeats`` after one warm-up)."""
-        best = float("inf")
+        logits of its last token: each of ``repeats`` runs after one warm-up."""
+        times: List[float] = []
         for i in range(repeats + 1):
             rid = ("prefill-timing", i)
             entry = StepEntry(rid, list(prompt), [len(prompt) - 1])
@@ -243,8 +271,8 @@ class Engine:
             dt = time.perf_counter() - t0
             self.runner.release(rid)
             if i:
-                best = min(best, dt)
-        return best
+                times.append(dt)
+        return times
 
     def time_decode(self, prompts: Sequence[Sequence[int]], steps: int, warmup: int) -> float:
         """Seconds of exactly ``steps`` decode steps of the batch ``prompts``

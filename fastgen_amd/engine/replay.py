@@ -17,6 +17,7 @@ from typing import IO, Optional
 import numpy as np
 import torch
 
+from ..config import read_config_json
 from .context import StepEntry
 from .model import Model
 from .runner import ModelRunner
@@ -25,14 +26,24 @@ DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, page_size: int = 64,
-           stdin: Optional[IO[str]] = None, stdout: Optional[IO[str]] = None, max_live: int = 4) -> int:
+           stdin: Optional[IO[str]] = None, stdout: Optional[IO[str]] = None, max_live: int = 4,
+           random_weights: Optional[int] = None) -> int:
     stdin = stdin or sys.stdin
     stdout = stdout or sys.stdout
     if not torch.cuda.is_available():
         raise RuntimeError("trace_run needs a GPU: fastgen_amd has no CPU execution path")
     out = Path(out_dir)
     out.mkdir(parents=True, exist_ok=True)
-    model = Model.from_folder(model_dir, DTYPES[dtype], "cuda:0")
+    if random_weights is None:
+        model = Model.from_folder(model_dir, DTYPES[dtype], "cuda:0")
+    else:  # the folder's (or the file's) configuration, tensors drawn on the device from the seed
+        path = Path(model_dir)
+        if path.is_file():
+            with open(path) as f:
+                config = json.load(f)
+        else:
+            config = read_config_json(path)
+        model = Model.random(config, random_weights, DTYPES[dtype], "cuda:0")
     # each request's count is rounded up to whole pages of at least 64 tokens
     unit = max(64, page_size)
     pool_tokens = -(-max_tokens // unit) * unit
@@ -47,6 +58,12 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, page_size:
             StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])])
             for e in rec.get("entries", [])
         ]
+        fresh = sum(1 for e in entries if not runner.cache.is_live(e.rid))
+        if fresh > runner.cache.free_slots():
+            raise RuntimeError(
+                f"step {step}: {len(runner.cache.live_requests()) + fresh} requests would be live, --max-live is"
+                f" {max_live}"
+            )
         if entries:
             logits = runner.step(entries)
             if logits is not None:
@@ -71,5 +88,12 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=64, help="tokens per cache page (default 64)")
+    ap.add_argument("--max-live", type=int, default=4, help="most requests that are live at a time (default 4)")
+    ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                    help="read no weights: --model names a folder with config.json (or the file itself), the"
+                         " tensors are drawn on the GPU from this seed")
     a = ap.parse_args(argv)
-    return replay(a.model, a.dtype, a.out, a.max_tokens, a.page_size)
+    if a.max_live < 1:
+        ap.error("--max-live must be at least 1")
+    return replay(a.model, a.dtype, a.out, a.max_tokens, a.page_size, max_live=a.max_live,
+                  random_weights=a.random_weights)

@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
-from ..cache.storage import CacheStorage, group_entries
+from ..cache.storage import CacheStorage, group_entries, tokens_for_free_memory
 from ..kernels.ops import upload
 from .context import StepContext, StepEntry, build_context, context_from_packed, pack_context
 from .model import Model
@@ -111,15 +111,20 @@ class ModelRunner:
     """A model with its cache: admits requests, steps them, lets them go.
 
     ``max_tokens`` is the number of tokens the pages of one group can hold
-    (each live request's length counts rounded up to whole pages);
-    ``max_requests`` is the number of state slots.
+    (each live request's length counts rounded up to whole pages); None: as
+    many as the device's free memory holds beside ``reserve_bytes``, at most
+    ``at_most_tokens``.  ``max_requests`` is the number of state slots.
     """
 
-    def __init__(self, model: Model, page_size: int = 64, max_tokens: int = 4096, max_requests: int = 64,
-                 pages_per_group: Optional[Sequence[int]] = None) -> None:
+    def __init__(self, model: Model, page_size: int = 64, max_tokens: Optional[int] = 4096, max_requests: int = 64,
+                 pages_per_group: Optional[Sequence[int]] = None, reserve_bytes: int = 2 << 30,
+                 at_most_tokens: Optional[int] = None) -> None:
         self.model = model
         self.page_size = page_size
         self.groups = group_entries(model.paged_needs())
+        if max_tokens is None and pages_per_group is None:
+            max_tokens = tokens_for_free_memory(self.groups, page_size, model.dtype, model.device, reserve_bytes,
+                                                at_most_tokens) if self.groups else page_size
         n_pages = -(-max_tokens // page_size)
         pages = list(pages_per_group) if pages_per_group is not None else [n_pages] * len(self.groups)
         self.cache = CacheManager(page_size, pages, [g.need.window for g in self.groups], max_requests)

@@ -57,6 +57,7 @@ class Request:
     # a request whose prompt and ``max_new`` tokens can never be held by the cache at once is
     # refused when it is added, unless it agrees to end early (reason ``max_seq``)
     truncate: bool = False
+    keep_stop_token: bool = True  # False: a stop id that ends the request is not part of what is reported
 
     def all_tokens(self) -> List[int]:
         return self.prompt + self.generated

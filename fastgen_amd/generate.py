@@ -44,7 +44,7 @@ class GenArgs:
     num_cuda_graphs: int = 64  # most captured decode steps (the reference: 16); 0: every step runs eagerly
     max_prefill: int = 8192  # token budget of one step
     prefill_gb: float = 0.5  # activation budget, used when sizing the cache
-    gpu_gb: float = 20  # memory budget, used when max_seq is negative
+    gpu_gb: float = 20  # memory budget, used when max_seq is negative; 0 or less: all that the GPU has free
     sync_freq: int = 10  # decode steps between host checks for finished requests (when nobody waits)
     seed: int = 777  # the reference's tools seed the global generator with 777 (tools/chat.py:47)
     dtype: torch.dtype = torch.bfloat16
@@ -59,6 +59,7 @@ class Packet:
     temperature: Optional[float] = None
     logprobs: Optional[List[float]] = None
     max_gen: Optional[int] = None
+    error: Optional[str] = None  # set on a packet that comes back refused (not in the reference)
 
 
 def cache_tokens_for_budget(model: Model, gen_args: GenArgs, bytes_per_token: int) -> int:
@@ -115,8 +116,6 @@ class Fastgen:
         on one GPU and takes None only."""
         if tp_mesh is not None:
             raise RuntimeError("fastgen_amd runs on one GPU: tp_mesh must be None")
-        if gen_args.host_cache_gb:
-            raise RuntimeError("fastgen_amd has no host-memory prefix cache: host_cache_gb must be 0")
         model_dir = loader.model_dir if isinstance(loader, HfLoader) else loader
         device_ = torch.device(device)
         if device_.type != "cuda":
@@ -125,19 +124,40 @@ class Fastgen:
         if stop_tokens is None and isinstance(loader, HfLoader):
             tokenizer = loader.load_tokenizer()
             stop_tokens = tokenizer.stop_tokens if tokenizer is not None else None
+        return cls.from_model(model, gen_args, stop_tokens)
+
+    @classmethod
+    def from_model(cls, model: Model, gen_args: GenArgs = GenArgs(),
+                   stop_tokens: Optional[Sequence[int]] = None, num_pages: Optional[int] = None) -> "Fastgen":
+        """Size the cache for a model that is already on the device (``fastgen/generate.py:206-244``):
+        ``num_pages`` pages if given, else ``max_seq`` tokens, else what ``gpu_gb`` leaves beside the
+        weights, else (``gpu_gb <= 0``) what the device has free."""
+        if gen_args.host_cache_gb:
+            raise RuntimeError("fastgen_amd has no host-memory prefix cache: host_cache_gb must be 0")
         if stop_tokens is None:
             eos = getattr(model.args, "extra", {}).get("eos_token_id", [])
             stop_tokens = eos if isinstance(eos, (list, tuple)) else [eos]
-        max_seq = gen_args.max_seq
-        if max_seq < 0:
-            esize = torch.empty((), dtype=gen_args.dtype).element_size()
-            per_token = sum(2 * n.n_kv_heads * n.head_dim * esize for n in model.paged_needs() if n is not None)
-            max_seq = cache_tokens_for_budget(model, gen_args, per_token)
-        max_batch = max(1, min(gen_args.max_batch, max_seq // gen_args.cache_block))  # generate.py:234-236
-        logger.info("cache of %d tokens in pages of %d, at most %d requests", max_seq, gen_args.cache_block, max_batch)
-        engine = Engine(model, page_size=gen_args.cache_block, max_tokens=max_seq, max_batch=max_batch,
-                        max_step_tokens=gen_args.max_prefill, max_seq=max_seq, seed=gen_args.seed,
-                        sync_freq=gen_args.sync_freq)
+        max_tokens: Optional[int] = gen_args.max_seq
+        if num_pages is not None:
+            if num_pages < 1:
+                raise ValueError("num_pages must be at least 1")
+            max_tokens = num_pages * gen_args.cache_block
+        elif gen_args.max_seq < 0:
+            if gen_args.gpu_gb > 0:
+                esize = torch.empty((), dtype=gen_args.dtype).element_size()
+                per_token = sum(2 * n.n_kv_heads * n.head_dim * esize for n in model.paged_needs() if n is not None)
+                max_tokens = cache_tokens_for_budget(model, gen_args, per_token)
+            else:
+                max_tokens = None  # the engine takes what is free
+        max_batch = gen_args.max_batch
+        if max_tokens is not None:
+            max_batch = max(1, min(max_batch, max_tokens // gen_args.cache_block))  # generate.py:234-236
+        engine = Engine(model, page_size=gen_args.cache_block, max_tokens=max_tokens, max_batch=max_batch,
+                        max_step_tokens=gen_args.max_prefill, max_seq=max_tokens, seed=gen_args.seed,
+                        sync_freq=gen_args.sync_freq, reserve_bytes=int(gen_args.prefill_gb * 1e9) + (2 << 30)
+                        if max_tokens is None else None)
+        logger.info("cache of %d tokens in pages of %d, at most %d requests",
+                    engine.scheduler.pool_tokens, gen_args.cache_block, engine.scheduler.max_batch)
         engine.runner.max_graphs = max(0, gen_args.num_cuda_graphs)
         return cls(engine, gen_args, stop_tokens)
 
@@ -147,8 +167,9 @@ class Fastgen:
         # the default (generate.py:790); greedy is the global switch (892)
         temp = (pkt.temperature or ga.temperature) if ga.use_sampling else 0.0
         max_gen = pkt.max_gen or ga.max_gen or (self.engine.scheduler.max_seq - len(pkt.tokens))
+        # maxlen = min(len + max_gen, max_seq) (generate.py:95-113): a request is cut short, not refused
         return SamplingParams(temperature=temp, top_p=ga.top_p, max_new_tokens=max(1, max_gen),
-                              stop_ids=self.stop_tokens, logprobs=ga.logprobs)
+                              stop_ids=self.stop_tokens, logprobs=ga.logprobs, truncate=True)
 
     def generate(self, q: "queue.Queue[Optional[Packet]]") -> Iterator[Packet]:
         """Packets from ``q`` in, finished packets out, in the order they
@@ -157,6 +178,7 @@ class Fastgen:
         when nothing is in flight (547)."""
         eoq = False
         pending = {}
+        refused: List[Packet] = []
         while True:
             while not eoq:
                 try:
@@ -166,8 +188,18 @@ class Fastgen:
                 if pkt is None:
                     eoq = True
                     break
-                rid = self.engine.add_request(pkt.tokens, self._params(pkt))
+                try:
+                    rid = self.engine.add_request(pkt.tokens, self._params(pkt))
+                except ValueError as e:
+                    # one caller's bad packet (empty, too long, an id outside the vocabulary) does not
+                    # end the others': it comes back at once, without tokens, the reason in ``error``
+                    logger.warning("packet %r refused: %s", pkt.thread_id, e)
+                    refused.append(Packet(thread_id=pkt.thread_id, tokens=[], temperature=pkt.temperature,
+                                          logprobs=None, max_gen=pkt.max_gen, error=str(e)))
+                    continue
                 pending[rid] = pkt
+            while refused:
+                yield refused.pop(0)
             if not self.engine.has_work():
                 if eoq:
                     return

@@ -24,10 +24,16 @@ from ..kernels import ops
 class SamplingParams:
     temperature: float = 0.0
     top_p: float = 1.0
-    seed: int = 0
+    seed: Optional[int] = None  # None: derived from the engine's seed and the request's arrival number
     max_new_tokens: int = 16
     stop_ids: Tuple[int, ...] = ()
     logprobs: bool = False
+    # whether a request that ends on a stop id keeps it as its last token (the reference's
+    # generator keeps it, fastgen/generate.py:647-662; its chat tool drops it, tools/chat.py:205-206)
+    keep_stop_token: bool = True
+    # a request whose prompt and max_new_tokens exceed the whole cache is refused, unless it
+    # agrees to end early (the reference clamps every request so, fastgen/generate.py:95-113)
+    truncate: bool = False
 
 
 class Sampler:

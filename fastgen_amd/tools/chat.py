@@ -5,6 +5,10 @@ quits, ``/r`` drops the last exchange); with one it generates once and exits:
 
     fgchat MODEL --prompt-ids 1,2,3 --max-tokens 32 --temperature 0
     fgchat MODEL --random-prompt 128 --max-tokens 64
+    fgchat --config config.json --random-weights 2 --random-prompt 128 --max-tokens 64 --num-pages 16
+
+``--random-weights SEED`` needs no weights on disk: the configuration comes from ``--config FILE`` (or from
+``config.json`` in MODEL) and the tensors are drawn on the GPU from the seed.
 """
 
 from __future__ import annotations
@@ -21,7 +25,8 @@ import torch
 
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="fgchat", description="Generate with a model folder on one MI355X.")
-    ap.add_argument("model", help="model folder (config.json, safetensors, optionally tokenizer.json)")
+    ap.add_argument("model", nargs="?", default=None,
+                    help="model folder (config.json, safetensors, optionally tokenizer.json)")
     ap.add_argument("--temperature", type=float, default=0.7, help="0 is greedy (default 0.7)")
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--max-tokens", type=int, default=None, help="most tokens to generate")
@@ -37,10 +42,20 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--max-seq", type=int, default=-1, help="cache size in tokens (default: from --gpu-gb)")
     ap.add_argument("--max-step-tokens", type=int, default=8192, help="token budget of one step")
+    ap.add_argument("--num-pages", type=int, default=None, help="cache size in pages (overrides --max-seq and --gpu-gb)")
+    ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                    help="no weights are read: they are drawn on the GPU from this seed")
+    ap.add_argument("--config", default=None, metavar="FILE",
+                    help="a config.json for --random-weights (default: the one in MODEL)")
+    ap.add_argument("--drop-stop-token", action="store_true",
+                    help="a stop id that ends the generation is not printed among the ids")
     return ap
 
 
 def main(argv: Optional[List[str]] = None) -> int:
+    import json
+
+    from ..engine import Model
     from ..generate import Fastgen, GenArgs, Packet
     from .tokenizer import FolderTokenizer
 
@@ -48,14 +63,34 @@ def main(argv: Optional[List[str]] = None) -> int:
     if a.tensor_parallel != 1:
         print("fgchat: this engine runs on one GPU; --tensor-parallel must be 1", file=sys.stderr)
         return 2
+    if a.model is None and (a.random_weights is None or a.config is None):
+        print("fgchat: give a model folder, or --random-weights SEED with --config FILE", file=sys.stderr)
+        return 2
+    if a.config is not None and a.random_weights is None:
+        print("fgchat: --config is for --random-weights; a model folder brings its own config.json", file=sys.stderr)
+        return 2
     logging.basicConfig(level=logging.INFO if a.verbose else logging.WARNING)
-    tokenizer = FolderTokenizer.maybe(a.model)
+    tokenizer = FolderTokenizer.maybe(a.model) if a.model is not None else None
     gen_args = GenArgs(
         use_sampling=bool(a.temperature), temperature=a.temperature, top_p=a.top_p, max_batch=1,
         max_gen=a.max_tokens, gpu_gb=a.gpu_gb, cache_block=a.page_size, max_seq=a.max_seq,
         max_prefill=a.max_step_tokens, seed=a.seed, dtype=getattr(torch, a.dtype),
     )
-    fg = Fastgen.build(a.model, gen_args, stop_tokens=tokenizer.stop_tokens if tokenizer else None)
+    stop_tokens = tokenizer.stop_tokens if tokenizer else None
+    if a.random_weights is not None:
+        from ..config import read_config_json
+
+        if a.config is not None:
+            with open(a.config) as f:
+                config = json.load(f)
+        else:
+            config = read_config_json(a.model)
+        model = Model.random(config, a.random_weights, gen_args.dtype, "cuda:0")
+        fg = Fastgen.from_model(model, gen_args, stop_tokens if stop_tokens is not None else (), a.num_pages)
+    elif a.num_pages is not None:
+        fg = Fastgen.from_model(Model.from_folder(a.model, gen_args.dtype, "cuda:0"), gen_args, stop_tokens, a.num_pages)
+    else:
+        fg = Fastgen.build(a.model, gen_args, stop_tokens=stop_tokens)
     q: "queue.Queue" = queue.Queue()
     gen = fg.generate(q)
 
@@ -80,6 +115,8 @@ def main(argv: Optional[List[str]] = None) -> int:
             g = torch.Generator().manual_seed(a.seed)
             ids = torch.randint(0, fg.engine.model.vocab_size, (a.random_prompt,), generator=g).tolist()
         out = run(ids)
+        if a.drop_stop_token and out and out[-1] in fg.stop_tokens:
+            out = out[:-1]
         print(",".join(str(t) for t in out))
         if tokenizer is not None:
             print(tokenizer.decode([t for t in out if t not in tokenizer.stop_tokens]))

@@ -82,7 +82,7 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: O
     G = H // KV
     out = torch.empty_like(q)
     scale = hd**-0.5
-    idx = torch.arange(T)
+    idx = torch.arange(T, device=q.device)
     mask = idx[None, :] <= idx[:, None]
     if window:
         mask &= idx[None, :] > idx[:, None] - window
@@ -116,11 +116,12 @@ def plain_forward(weights: Mapping[str, torch.Tensor], config: Mapping, tokens, 
     hd = D // H  # fastgen/forward.py:364
     eps = config["rms_norm_eps"]
     L = config["num_hidden_layers"]
-    freqs = plain_rope_frequencies(hd, config["rope_theta"], config.get("rope_scaling"))
+    dev = next(iter(weights.values())).device  # where the weights are is where it runs (the CPU, in most tests)
+    freqs = plain_rope_frequencies(hd, config["rope_theta"], config.get("rope_scaling")).to(dev)
     W = {k: v.to(dtype) for k, v in weights.items()}
-    tok = torch.as_tensor(tokens, dtype=torch.long)
+    tok = torch.as_tensor(tokens, dtype=torch.long, device=dev)
     T = tok.numel()
-    pos = torch.arange(T)
+    pos = torch.arange(T, device=dev)
     h = W["model.embed_tokens.weight"][tok]  # forward.py:406-409
     for i in range(L):
         p = f"model.layers.{i}."

@@ -219,3 +219,64 @@ def test_unsharpened_model_and_loader_round_trip(tmp_path):
     runner = make_runner(folder, torch.float32, 16, 128)
     got = run_trace(runner, traces.chunks({"x": 87}), toks)
     assert_close(got, want, torch.float32, None, "written folder")
+
+
+def test_trace_run_with_random_weights_and_more_live_requests(tmp_path):
+    """``--random-weights SEED``: a folder with config.json alone (or the file) is enough; the same
+    seed gives the same logits however the tokens are cut (bit for bit in 32-bit).  ``--max-live``:
+    six requests live at once; a seventh is refused with a message that names the option."""
+    cfg = tmp_path / "cfg"
+    cfg.mkdir()
+    (cfg / "config.json").write_text(json.dumps(TINY_A))
+    toks = {f"r{i}": [(7 * i + 3 * j) % 256 for j in range(20 + i)] for i in range(6)}
+
+    def run(lines, out, *more):
+        cmd = [sys.executable, str(REPO / "bin" / "trace_run"), "--model", str(cfg), "--dtype", "float32", "--out",
+               str(out), "--max-tokens", str(6 * 64), "--page-size", "16", "--random-weights", "5", *more]
+        return subprocess.run(cmd, input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True,
+                              text=True, timeout=600)
+
+    whole = [{"step": 0, "entries": [{"id": r, "tokens": t, "want": [len(t) - 1]} for r, t in toks.items()],
+              "end": list(toks)}]
+    cut = [{"step": 0, "entries": [{"id": r, "tokens": t[:7], "want": []} for r, t in toks.items()], "end": []},
+           {"step": 1, "entries": [{"id": r, "tokens": t[7:], "want": [len(t) - 8]} for r, t in toks.items()],
+            "end": list(toks)}]
+    p = run(whole, tmp_path / "a", "--max-live", "6")
+    assert p.returncode == 0, p.stderr[-2000:]
+    p = run(cut, tmp_path / "b", "--max-live", "6")
+    assert p.returncode == 0, p.stderr[-2000:]
+    a = np.fromfile(tmp_path / "a" / "0.f32", dtype="<f4").reshape(6, 256)
+    b = np.fromfile(tmp_path / "b" / "1.f32", dtype="<f4").reshape(6, 256)
+    assert np.isfinite(a).all() and np.array_equal(a, b) and np.abs(a).max() > 0
+    assert len({tuple(row) for row in a.round(4).tolist()}) == 6  # six requests, six different rows
+    p = run(whole, tmp_path / "c", "--model", str(cfg / "config.json"))  # the default: four live requests
+    assert p.returncode != 0 and "--max-live is 4" in p.stderr
+
+
+@pytest.mark.parametrize("n_live,captured", [(24, False), (24, True), (61, False), (61, True)])
+def test_many_requests_decode_together_bfloat16(n_live, captured, tmp_path):
+    """Dozens of live requests of different lengths, prompts fed in portions, then 45 decode steps
+    of all of them together: the split and combine attention kernels with dozens of items, the wide
+    products at 17..64 rows, and (captured) the recorded step with a batch filled up to its capacity
+    (61 -> 64) by stand-in sequences.  Every position against the plain implementation."""
+    cfg = TINY_C
+    weights = sharpen(plain_random_weights(cfg, 8))
+    weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    folder = save_model_folder(tmp_path / "many", cfg, weights)
+    rng = np.random.default_rng(n_live)
+    n_decode = 45
+    prompts = {f"r{i}": int(n) for i, n in enumerate(rng.integers(1, 300, n_live))}
+    prompts["r0"], prompts["r1"] = 1, 460  # the shortest there is, and one far longer than the others
+    g = torch.Generator().manual_seed(12)
+    tokens = {rid: torch.randint(0, cfg["vocab_size"], (n + n_decode,), generator=g).tolist()
+              for rid, n in prompts.items()}
+    trace = traces.many_decoding_together(prompts, n_decode, seed=n_live)
+    runner = make_runner(folder, torch.bfloat16, 16, traces.max_live_tokens(trace, 64), max_requests=n_live)
+    runner.use_graphs = captured
+    got = run_trace(runner, trace, tokens)
+    assert runner.cache.live_requests() == []
+    assert bool(runner.graphs) == captured
+    if captured:
+        assert {c for c, _ in runner.graphs} == {24 if n_live == 24 else 64}
+    assert_close(got, plain_logits(weights, cfg, tokens), torch.bfloat16,
+                 plain_logits(weights, cfg, tokens, torch.bfloat16), f"{n_live} live")

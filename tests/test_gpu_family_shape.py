@@ -36,7 +36,7 @@ def family(tmp_path_factory):
              for r, t in tokens.items()}
     plain32 = plain_logits(w, FAMILY, tokens)
     noise16 = plain_logits(w, FAMILY, tokens, torch.bfloat16)
-    return dict(folder=folder, tokens=tokens, exact=exact, plain32=plain32, noise16=noise16)
+    return dict(folder=folder, tokens=tokens, exact=exact, plain32=plain32, noise16=noise16, weights=w)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -50,3 +50,37 @@ def test_family_shape_under_every_cut(family, dtype):
             assert_close(got, family["exact"], dtype, family["plain32"], name)
         else:
             assert_close(got, family["plain32"], dtype, family["noise16"], name)
+
+
+@pytest.mark.parametrize("n_live", [24, 61])
+def test_family_shape_many_requests_decode_together(family, n_live):
+    """The benchmark's decode path at its layer sizes: dozens of live requests of different lengths,
+    prompts fed in portions, then 40 decode steps of all together, eagerly and from captured steps
+    (61 requests in a step recorded for 64): the wide products with k splits at 17..64 rows, the
+    library's q/k/v product with the rotation kernel, split attention with dozens of items and both
+    combine kernels.  Every position against the plain implementation, which for this many tokens
+    runs its torch operations on the GPU; that run is pinned to the CPU run on one request."""
+    import numpy as np
+
+    w_gpu = {k: v.to("cuda:0") for k, v in family["weights"].items()}
+    pin = plain_forward(w_gpu, FAMILY, family["tokens"]["b"]).cpu()
+    assert torch.allclose(pin, family["plain32"]["b"], atol=1e-4 * float(pin.abs().max()), rtol=0)
+    rng = np.random.default_rng(n_live)
+    n_decode = 40
+    prompts = {f"r{i}": int(n) for i, n in enumerate(rng.integers(1, 150, n_live))}
+    prompts["r0"], prompts["r1"] = 1, 700
+    g = torch.Generator().manual_seed(n_live)
+    tokens = {r: torch.randint(0, FAMILY["vocab_size"], (n + n_decode,), generator=g).tolist()
+              for r, n in prompts.items()}
+    want = {r: plain_forward(w_gpu, FAMILY, t).cpu() for r, t in tokens.items()}
+    noise = {r: plain_forward(w_gpu, FAMILY, t, torch.bfloat16).cpu() for r, t in tokens.items()}
+    del w_gpu
+    trace = traces.many_decoding_together(prompts, n_decode, seed=n_live, budget=256)
+    for captured in (False, True):
+        runner = make_runner(family["folder"], torch.bfloat16, 64, traces.max_live_tokens(trace, 64),
+                             max_requests=n_live)
+        runner.use_graphs = captured
+        got = run_trace(runner, trace, tokens)
+        assert bool(runner.graphs) == captured
+        assert_close(got, want, torch.bfloat16, noise, f"{n_live} live, captured={captured}")
+        del runner

@@ -437,5 +437,122 @@ def test_bench_line():
     assert j["n_gpus"] == 1 and j["steps"] == 3 and j["warmup"] == 1 and j["dtype"] == "bf16" and j["value"] > 0
     assert j["config"]["layers"] == 1 and j["config"]["layers_full"] == 32 and len(j["config"]) <= 20
     assert all(not isinstance(v, (dict, list)) for v in j["config"].values())
-    assert set(j["prefill"]) == {"value", "tokens", "ms", "frac"} and j["prefill"]["tokens"] == 2048
+    assert set(j["prefill"]) >= {"value", "tokens", "ms", "frac"} and j["prefill"]["tokens"] == 2048
+    assert j["prefill"]["repeats"] >= 3 and j["prefill"]["best_ms"] <= j["prefill"]["ms"]
+    # the capacity that the line names is the capacity that the cache has
+    assert j["config"]["seq_len"] == 8192 and j["config"]["cache_tokens"] == 8 * 8192
     assert j["roofline"]["bound"] == "hbm" and j["roofline"]["peak"] == 8000.0 and 0 < j["roofline"]["frac"] < 1
+
+
+def test_stop_token_kept_or_dropped_and_seed_zero(tiny_b):
+    """``keep_stop_token=False`` reports the request without the stop id that ended it (the
+    reference's generator keeps it, its chat tool drops it); seed 0 is a seed like any other."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=1024, max_batch=4)
+    prompt = tiny_b["prompts"][1]
+    free = plain_greedy(tiny_b["weights"], TINY_B, prompt, 10)
+    stop = free[4]
+    cut = free.index(stop)
+    for overlap in (True, False):
+        eng.overlap_steps = overlap
+        kept, dropped = eng.generate([prompt] * 2, [
+            SamplingParams(max_new_tokens=10, stop_ids=(stop,), logprobs=True),
+            SamplingParams(max_new_tokens=10, stop_ids=(stop,), keep_stop_token=False, logprobs=True)])
+        assert kept == free[: cut + 1] and dropped == free[:cut]
+    # max_new_tokens reached on the very token that is a stop id: it is dropped all the same
+    assert eng.generate([prompt], SamplingParams(max_new_tokens=cut + 1, stop_ids=(stop,), keep_stop_token=False)) \
+        == [free[:cut]]
+    # seeds: 0 is a seed of its own, None derives one from the engine's seed and the arrival number
+    hot = lambda seed: SamplingParams(temperature=1.5, max_new_tokens=12, seed=seed)
+    a = eng.generate([prompt], hot(0))
+    b = eng.generate([prompt], hot(0))
+    c = eng.generate([prompt], hot(None))
+    d = eng.generate([prompt], hot(None))
+    e = eng.generate([prompt], hot(1))
+    assert a == b and c != d and a != e
+
+
+def test_a_request_that_never_fits_is_refused_or_cut(tiny_b):
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=128, max_batch=2)
+    prompt = tiny_b["prompts"][3]  # 90 tokens
+    with pytest.raises(ValueError, match="can never fit"):
+        eng.generate([tiny_b["prompts"][1], prompt], SamplingParams(max_new_tokens=40))
+    assert not eng.has_work() and eng.runner.cache.live_requests() == []  # all or nothing
+    out = eng.generate([prompt], SamplingParams(max_new_tokens=40, truncate=True))[0]
+    assert out == plain_greedy(tiny_b["weights"], TINY_B, prompt, 38)  # 90 + 38 = the 128 tokens of the cache
+
+
+def test_a_refused_packet_comes_back_and_the_others_go_on(tiny_b):
+    from fastgen_amd.generate import Fastgen, GenArgs, Packet
+
+    fg = Fastgen.build(tiny_b["folder"], GenArgs(use_sampling=False, max_batch=3, max_seq=256, max_gen=6,
+                                                cache_block=32, dtype=torch.float32), stop_tokens=())
+    q = queue.Queue()
+    q.put(Packet(thread_id="good0", tokens=tiny_b["prompts"][1]))
+    q.put(Packet(thread_id="empty", tokens=[]))
+    q.put(Packet(thread_id="alien", tokens=[1, 2, 10**6]))
+    q.put(Packet(thread_id="long", tokens=[1] * 300))
+    q.put(Packet(thread_id="good1", tokens=tiny_b["prompts"][2]))
+    q.put(None)
+    out = {p.thread_id: p for p in fg.generate(q)}
+    assert set(out) == {"good0", "empty", "alien", "long", "good1"}
+    for bad in ("empty", "alien", "long"):
+        assert out[bad].tokens == [] and out[bad].error
+    assert out["good0"].error is None
+    assert out["good0"].tokens == plain_greedy(tiny_b["weights"], TINY_B, tiny_b["prompts"][1], 6)
+    assert out["good1"].tokens == plain_greedy(tiny_b["weights"], TINY_B, tiny_b["prompts"][2], 6)
+    assert fg.engine.runner.cache.live_requests() == []
+
+
+def test_cache_sized_to_the_memory_that_is_free(tiny_b):
+    """``max_tokens=None``: the cache takes what the device has free beside a reserve, in whole
+    pages, and never more than all requests at their longest can use."""
+    from fastgen_amd.engine import Engine, Model
+    from fastgen_amd.generate import Fastgen, GenArgs
+
+    model = Model.from_folder(tiny_b["folder"], torch.bfloat16, "cuda:0")
+    eng = Engine(model, page_size=32, max_tokens=None, max_batch=3)
+    assert eng.scheduler.pool_tokens == 3 * 256  # max_position_embeddings 256 a request: no more is ever needed
+    del eng
+    torch.cuda.empty_cache()
+    free = torch.cuda.mem_get_info()[0] + torch.cuda.memory_reserved() - torch.cuda.memory_allocated()
+    per_token = 2 * 3 * 32 * 2 * 3  # K and V, 3 kv heads of 32, bfloat16, 3 layers
+    reserve = free - 1000 * per_token - 17  # room for 1,000 tokens and a bit
+    eng = Engine(model, page_size=32, max_tokens=None, max_batch=64, reserve_bytes=reserve)
+    assert eng.scheduler.pool_tokens == 992  # whole pages
+    with pytest.raises(RuntimeError, match="no room for one cache page"):
+        Engine(model, page_size=32, max_tokens=None, max_batch=64, reserve_bytes=free + (1 << 30))
+    fg = Fastgen.from_model(model, GenArgs(gpu_gb=0, max_batch=2, cache_block=32))
+    assert fg.engine.scheduler.pool_tokens == 2 * 256
+    fg = Fastgen.from_model(model, GenArgs(max_batch=2, cache_block=32), num_pages=5)
+    assert fg.engine.scheduler.pool_tokens == 160
+
+
+def test_command_line_with_random_weights_and_pages(tiny_b, tmp_path):
+    """``fgchat --config FILE --random-weights SEED --num-pages N``: no weights on disk; the same
+    seed gives the same tokens, another seed other tokens; the cache has the pages asked for."""
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(TINY_B))
+    base = [sys.executable, str(REPO / "bin" / "fgchat"), "--config", str(cfg), "--prompt-ids", "5,6,7,8",
+            "--max-tokens", "12", "--temperature", "0", "--dtype", "float32", "--page-size", "16", "--verbose"]
+
+    def run(*more):
+        proc = subprocess.run(base + list(more), capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        return [int(x) for x in proc.stdout.strip().splitlines()[0].split(",")], proc.stderr
+
+    a, log = run("--random-weights", "3", "--num-pages", "4")
+    assert "cache of 64 tokens in pages of 16" in log
+    b, _ = run("--random-weights", "3", "--num-pages", "4")
+    c, _ = run("--random-weights", "4", "--num-pages", "4")
+    assert a == b and a != c and len(a) == 12
+    # 2 pages of 16: the prompt's 4 tokens and 28 more fit; the reference's clamp cuts the generation short
+    d, _ = run("--random-weights", "3", "--num-pages", "2", "--max-tokens", "100")
+    assert len(d) == 28 and d[:12] == a
+    proc = subprocess.run(base[:2] + ["--prompt-ids", "1"], capture_output=True, text=True, timeout=60)
+    assert proc.returncode == 2 and "--random-weights" in proc.stderr

@@ -91,3 +91,29 @@ def max_live_tokens(trace: List[Step], round_to: int = 64) -> int:
         for rid in ends:
             held.pop(rid, None)
     return worst
+
+
+def many_decoding_together(prompt_lens: Dict[str, int], n_decode: int, seed: int = 0, budget: int = 96,
+                           max_per_step: int = 6) -> List[Step]:
+    """All requests become live, their prompts fed in portions of changing size (a few requests a
+    step, under a token budget); then every request decodes, all of them in every step, for
+    ``n_decode`` steps, and all end together."""
+    rng = random.Random(seed)
+    fed = {rid: 0 for rid in prompt_lens}
+    steps: List[Step] = []
+    while any(fed[r] < n for r, n in prompt_lens.items()):
+        entries, left = [], budget
+        todo = [r for r, n in prompt_lens.items() if fed[r] < n]
+        rng.shuffle(todo)
+        for rid in todo[:max_per_step]:
+            c = min(prompt_lens[rid] - fed[rid], rng.choice([2, 3, 7, 16, 33, 64]), left)
+            if c < 1:
+                break
+            entries.append((rid, fed[rid], c))
+            fed[rid] += c
+            left -= c
+        steps.append((entries, []))
+    for s in range(n_decode):
+        steps.append(([(rid, n + s, 1) for rid, n in prompt_lens.items()],
+                      list(prompt_lens) if s == n_decode - 1 else []))
+    return steps
