@@ -25,6 +25,9 @@
 // Semantics as in attention.hip (fastgen/forward.py:176-258).
 #include "common.h"
 #include "kv_layout.h"
+#include "attention_static.h"
+
+#include <stdio.h>
 
 #ifndef FG_HD
 #error "compile with -DFG_HD=<head size>"
@@ -647,6 +650,88 @@ extern "C" int fg_attn_split(const void* q, int q_stride, void* out, int out_str
     attn_combine_kernel<<<dim3(n_kv, max_chunks), 256, 0, stream>>>(
         part_o, part_ml, plan, (bf16_t*)out, out_stride, n_heads, n_kv);
   return fg_launch_status();
+}
+
+// ----------------------------------------------------------- without allocation
+// The plan, part_o and part_ml of a call live in this array (see attention_static.h).  In host code
+// the array's name is only a handle for hipGetSymbolAddress: each GPU has its own copy at its own
+// address, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[FG_ATTN_STATIC_BYTES];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static unsigned char* scratch_ptr[STATIC_MAX_DEVICES];  // the array's address on each device, once known
+static thread_local char static_error[256] = "";
+
+extern "C" const char* fg_attn_decode_static_error() { return static_error; }
+
+// bytes of scratch for max_chunks chunks: the plan (rounded up to 256 bytes), then part_o, then part_ml
+static size_t static_plan_bytes(int max_chunks) {
+  return (((size_t)(PLAN_HEAD + 8LL * max_chunks) * sizeof(int)) + 255) / 256 * 256;
+}
+static size_t static_bytes(int max_chunks, int n_kv) {
+  return static_plan_bytes(max_chunks) + (size_t)max_chunks * n_kv * 16 * (HD + 2) * sizeof(float);
+}
+
+extern "C" int fg_attn_decode_static_max_chunks(int n_kv) {
+  if (n_kv <= 0) return 0;
+  int lo = 0, hi = 65535;  // the largest count whose scratch fits
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (static_bytes(mid, n_kv) <= FG_ATTN_STATIC_BYTES) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// The address of `scratch` on the current device (nullptr, with the reason in static_error, if it
+// cannot be had).
+static unsigned char* static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) {
+    snprintf(static_error, sizeof static_error, "fg_attn_decode_static: no current device (%s, device %d)",
+             hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  unsigned char* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p) return p;
+  e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) {
+    snprintf(static_error, sizeof static_error, "fg_attn_decode_static: hipGetSymbolAddress failed on device %d: %s",
+             dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);  // every thread finds the same address
+  return p;
+}
+
+extern "C" int fg_attn_decode_static(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                                     const void* v_pages, const int* block_table, int bt_stride, const int* items,
+                                     int n_items, int max_chunks, int min_tiles, int max_rows, int n_heads,
+                                     int n_kv, int hd, int page_size, float scale, int window,
+                                     hipStream_t stream) {
+  static_error[0] = 0;
+  if (n_items <= 0) return FG_OK;
+  if (n_kv <= 0 || max_chunks < 2 * n_items || static_bytes(max_chunks, n_kv) > FG_ATTN_STATIC_BYTES) {
+    snprintf(static_error, sizeof static_error,
+             "fg_attn_decode_static: %d items in %d chunks for %d kv heads of size %d need %zu bytes of scratch, "
+             "the static array holds %u (at most %d chunks, half as many items)",
+             n_items, max_chunks, n_kv, HD, n_kv > 0 ? static_bytes(max_chunks, n_kv) : (size_t)0,
+             FG_ATTN_STATIC_BYTES, fg_attn_decode_static_max_chunks(n_kv));
+    return n_kv > 0 && max_chunks >= 2 * n_items ? FG_ERR_SCRATCH : FG_ERR_ARG;
+  }
+  unsigned char* base = static_scratch();
+  if (!base) return FG_ERR_SCRATCH;
+  int* plan = (int*)base;
+  float* part_o = (float*)(base + static_plan_bytes(max_chunks));
+  float* part_ml = part_o + (size_t)max_chunks * n_kv * 16 * HD;
+  int st = fg_attn_plan(items, n_items, window, max_chunks, min_tiles, plan, stream);
+  if (st == FG_OK)
+    st = fg_attn_split(q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_stride, plan, n_items,
+                       max_chunks, max_rows, part_o, part_ml, n_heads, n_kv, hd, page_size, scale, window, stream);
+  if (st != FG_OK)
+    snprintf(static_error, sizeof static_error, "fg_attn_decode_static: %s",
+             st == FG_ERR_ARG ? "an argument that the kernels cannot take" : "a kernel launch failed");
+  return st;
 }
 
 // ------------------------------------------------------------------- tile

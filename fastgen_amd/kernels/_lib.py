@@ -33,7 +33,7 @@ HIPCC_FLAGS = [
     # packed fp32 instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-HEADERS = ["common.h", "kv_layout.h"]
+HEADERS = ["common.h", "kv_layout.h", "attention_static.h"]
 
 # library name -> source file
 LIBRARIES: Dict[str, str] = {
