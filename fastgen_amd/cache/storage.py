@@ -8,8 +8,9 @@ reference keeps per layer ``[n_pages*P, KV, hd]`` for both,
 ``fastgen/cache.py:66-78``.)  Pages are not cleared when they change hands:
 what a page holds beyond a request's length is never read.
 
-Per-request state of fixed size lives in ``[n_slots, *shape]`` tensors, one
-per run entry that asked for it, cleared when a slot is handed out.
+Per-request state of fixed size lives in ``[n_slots + 1, *shape]`` tensors, one
+per run entry that asked for it, cleared when a slot is handed out (the last
+row is nobody's: stand-in sequences of a captured step use it).
 """
 
 from __future__ import annotations
@@ -82,8 +83,11 @@ class CacheStorage:
             self.v.append(torch.empty((n, n_pages, kv, hd, page_size), dtype=dtype, device=device))
             for j, e in enumerate(grp.entries):
                 self._where[e] = (g, j)
+        # one row more than there are slots: row ``n_slots`` belongs to nobody.  The stand-in sequences that
+        # fill a captured step up to its capacity keep their state there, so that no request's state moves.
+        self.scratch_slot = n_slots
         self.state: Dict[int, torch.Tensor] = {
-            e: torch.zeros((n_slots, *need.shape), dtype=need.dtype, device=device)
+            e: torch.zeros((n_slots + 1, *need.shape), dtype=need.dtype, device=device)
             for e, need in state_needs.items()
         }
 

@@ -29,13 +29,17 @@ class PartSpec:
 @dataclass(frozen=True)
 class LayerSpec:
     """One layer: a token mixer and a feed-forward, each with its norm, and
-    the name of the arrangement that wires them to the residual stream."""
+    the name of the arrangement that wires them to the residual stream.
+    ``extra_norms``: further norms by name, for arrangements that own more
+    than two (norms after the mixer and the feed-forward, say); the
+    arrangement gets them as a dict."""
 
     mixer: PartSpec
     ffn: PartSpec
     mixer_norm: PartSpec
     ffn_norm: PartSpec
     arrangement: str = "pre_norm"
+    extra_norms: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

@@ -1042,6 +1042,5 @@ extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stri
   return fg_launch_status();
 }
 
-extern "C" int fg_attn_head_dim() { return HD; }
 // query rows (tokens x heads of a kv head's group) of one item of fg_attn_tile
 extern "C" int fg_attn_tile_rows() { return TILE_ROWS; }

@@ -232,20 +232,6 @@ extern "C" int fg_rmsnorm(const void* x, const void* w, void* out, int n_rows, i
 // 8: columns 16k .. 16k+7 are gate 8k .. 8k+7, columns 16k+8 .. 16k+15 their up
 // values (the row order in which the gate/up matrix is kept, so that one tile
 // of a matrix product holds both).  hidden % 8 == 0.
-template <class TA>
-__global__ __launch_bounds__(ROWS_THREADS) void silu_mul_kernel(
-    const TA* __restrict__ gu, TA* __restrict__ out, int hidden) {
-  const TA* row = gu + (size_t)blockIdx.y * 2 * hidden;
-  TA* o = out + (size_t)blockIdx.y * hidden;
-  const int i = blockIdx.x * ROWS_THREADS + threadIdx.x;
-  if (i < hidden) {
-    const int col = 16 * (i / 8) + i % 8;
-    const float gv = to_f<TA>(row[col]);
-    const float uv = to_f<TA>(row[col + 8]);
-    o[i] = from_f<TA>(gv / (1.f + expf(-gv)) * uv);
-  }
-}
-
 // eight elements a thread, for hidden % 8 == 0
 template <class TA>
 __global__ __launch_bounds__(ROWS_THREADS) void silu_mul_vec_kernel(
@@ -273,19 +259,16 @@ extern "C" int fg_silu_mul(const void* gu, void* out, int n_rows, int hidden, in
   // blockIdx.y is limited to 65535: rows beyond that go to further launches
   for (int r0 = 0; r0 < n_rows; r0 += 65535) {
     const int nr = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
-    const bool vec = true;  // hidden % 8 == 0 is required by the interleaved layout
-    const int per_block = vec ? ROWS_THREADS * 8 : ROWS_THREADS;
+    const int per_block = ROWS_THREADS * 8;  // (hidden % 8 == 0 is what the interleaved layout asks for anyway)
     dim3 grid((hidden + per_block - 1) / per_block, nr);
     if (act_dtype == FG_F32) {
       const float* g = (const float*)gu + (size_t)r0 * 2 * hidden;
       float* o = (float*)out + (size_t)r0 * hidden;
-      if (vec) silu_mul_vec_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
-      else silu_mul_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+      silu_mul_vec_kernel<float><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
     } else if (act_dtype == FG_BF16) {
       const bf16_t* g = (const bf16_t*)gu + (size_t)r0 * 2 * hidden;
       bf16_t* o = (bf16_t*)out + (size_t)r0 * hidden;
-      if (vec) silu_mul_vec_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
-      else silu_mul_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
+      silu_mul_vec_kernel<bf16_t><<<grid, ROWS_THREADS, 0, stream>>>(g, o, hidden);
     } else {
       return FG_ERR_ARG;
     }

@@ -81,8 +81,9 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
     tables have that many columns whatever the requests hold, so that steps of
     the same batch shape have the same layout.  With ``pad_to`` the batch is
     filled up to that many sequences with stand-ins of one token at position 0
-    that write nothing to the cache (slot -1) and own no page (their block
-    table rows name page 0, which they only read): a captured step of
+    that write nothing to the cache (slot -1), own no page (their block
+    table rows name page 0, which they only read) and have the state row
+    behind the last slot, which is nobody's: a captured step of
     ``pad_to`` sequences then serves any smaller batch; the stand-ins' logits
     are the last rows and mean nothing."""
     n_real = len(entries)
@@ -108,7 +109,8 @@ def pack_context(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: 
                 raise ValueError(f"request {e.rid!r}: wanted place {w} is outside its {q_lens[b]} tokens")
             out_rows.append(int(q_start[b]) + int(w))
     out_rows += [int(q_start[b]) for b in range(n_real, B)]
-    slot_ids = np.array([cache.slot(e.rid) for e in entries] + [0] * n_pad, dtype=np.int32)
+    # stand-ins keep their state in the row behind the last slot, which belongs to no request
+    slot_ids = np.array([cache.slot(e.rid) for e in entries] + [cache.n_slots] * n_pad, dtype=np.int32)
 
     # one record per sequence (sequence, first flat token, tokens, first position): the items of the
     # attention kernels when every sequence brings so few tokens that it is one item; first in the

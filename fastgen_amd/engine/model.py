@@ -46,9 +46,11 @@ def build_parts(layout: ModelLayout) -> ModelParts:
         ffn = build_part("feed_forward", ls.ffn)
         n1 = build_part("norm", ls.mixer_norm)
         n2 = build_part("norm", ls.ffn_norm)
-        blocks.append(build_part("arrangement", PartSpec(ls.arrangement), mixer, ffn, n1, n2))
+        extra = {name: build_part("norm", spec) for name, spec in ls.extra_norms.items()}
+        # an arrangement that asks for no further norms is built from the four parts alone
+        blocks.append(build_part("arrangement", PartSpec(ls.arrangement), mixer, ffn, n1, n2, *([extra] if extra else [])))
         mixers.append(mixer)
-        parts += [mixer, ffn, n1, n2]
+        parts += [mixer, ffn, n1, n2, *extra.values()]
     final_norm = build_part("norm", layout.final_norm)
     head = build_part("head", layout.head)
     parts += [final_norm, head]

@@ -59,7 +59,7 @@ class _DecodeGraph:
 
     def __init__(self, runner: "ModelRunner", entries: Sequence[StepEntry], table_width: int) -> None:
         model, cache = runner.model, runner.cache
-        self.capacity = graph_capacity_for(len(entries))
+        self.capacity = runner.graph_capacity(len(entries))
         self.table_width = table_width
         packed, offs, shapes, host = pack_context(entries, cache, model.vocab_size, table_width, self.capacity)
         self.layout = (tuple(int(o) for o in offs), tuple(shapes))
@@ -71,12 +71,18 @@ class _DecodeGraph:
         self.packed = self.staging[0].to(model.device)
         self.ctx = context_from_packed(self.packed, offs, shapes, host, cache.page_size, model.dtype)
         self.ctx.graph_capacity = table_width * cache.page_size  # the longest sequence this step may meet
-        # warm up outside the capture (libraries load, the matrix library picks its kernels), then capture
+        # warm up outside the capture (libraries load, the matrix library picks its kernels), then capture.
+        # The warm-up is a step of its own: keys and values that it writes are the ones the replay writes
+        # again, but state of fixed size would move twice, so the rows of this step's slots are put back.
+        rows = self.ctx.slot_ids.long()
+        kept = {e: t.index_select(0, rows) for e, t in runner.storage.state.items()}
         side = torch.cuda.Stream(device=model.device)
         side.wait_stream(torch.cuda.current_stream(model.device))
         with torch.cuda.stream(side):
             model.forward(self.ctx, runner.stores)
         torch.cuda.current_stream(model.device).wait_stream(side)
+        for e, t in runner.storage.state.items():
+            t.index_copy_(0, rows, kept[e])
         torch.cuda.synchronize(model.device)
         # what the warm-up derived from this step's values (tables of sines, ...) is derived again
         # inside the capture, so that a replay derives it from its own values
@@ -134,14 +140,13 @@ class ModelRunner:
             self.storage.store_for(i, e.reads_cache_of) for i, e in enumerate(model.layout.order)
         ]
         self.last_context: Optional[StepContext] = None
-        # decode graphs: FG_NO_GRAPHS=1 switches them off (the reference: FG_NO_CUDA_GRAPHS)
-        # a mixer with state of its own is stepped eagerly: the warm-up run before a capture would
-        # advance its state twice
-        self.use_graphs = (os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and not model.state_needs()
-                           and model.capturable())
+        # decode graphs: FG_NO_GRAPHS=1 switches them off (the reference: FG_NO_CUDA_GRAPHS); a model with a
+        # part that cannot be recorded is stepped eagerly
+        self.use_graphs = os.environ.get("FG_NO_GRAPHS", "0") in ("", "0") and model.capturable()
         self.table_width = max(1, max(pages, default=1))
         self.graphs: Dict[Tuple[int, int], _DecodeGraph] = {}  # (capacity, table width) -> step, oldest use first
         self.graph_pool = None
+        self.graph_capacity = graph_capacity_for  # batch size -> sequences of the recorded step that serves it
         self.max_graphs = 64
         self.run_ahead = 16  # steps the host may prepare before the device has run them
 
@@ -225,7 +230,7 @@ class ModelRunner:
         """The captured step for these entries (whose pages are reserved): by batch capacity and
         block-table width.  At most ``max_graphs`` are kept; the one unused longest gives way."""
         held = max(self.cache.n_table_entries(e.rid, g) for e in entries for g in range(self.cache.n_groups))
-        key = (graph_capacity_for(len(entries)), graph_table_width_for(held, self.table_width))
+        key = (self.graph_capacity(len(entries)), graph_table_width_for(held, self.table_width))
         g = self.graphs.pop(key, None)
         if g is None:
             while len(self.graphs) >= self.max_graphs:

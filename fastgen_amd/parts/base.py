@@ -80,9 +80,14 @@ class Part:
 
     ``capturable``: whether ``forward`` may be recorded into a HIP graph, that
     is, whether it launches the same kernels with the same arguments whatever
-    the values on the device are.  A part that looks at device data on the
-    host (shapes that depend on the data) sets it to False; a model with such
-    a part is always stepped eagerly."""
+    the values on the device are, and takes everything that changes from step
+    to step (tokens, positions, lengths, block tables, slot ids) from the
+    context's device tensors.  A part that looks at device data on the host
+    (shapes that depend on the data), or that uses the context's host copies
+    in a step of one token a sequence, sets it to False; a model with such a
+    part is always stepped eagerly.  Only steps in which every sequence brings
+    one token are recorded; a recorded step may hold stand-in sequences, whose
+    state slot (``ctx.slot_ids``) is a row that belongs to no request."""
 
     capturable: bool = True
 

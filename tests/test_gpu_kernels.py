@@ -520,7 +520,7 @@ def test_kernels_refuse_what_they_cannot_take(ops):
 CUTS = {"auto": (None, 4), "coarse": ("least", 4), "fine": (4096, 1), "pairs": (4096, 2)}
 
 
-def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto"):
+def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto", max_rows=16):
     import numpy as np
 
     q_lens = [b for _, b in seqs]
@@ -533,7 +533,7 @@ def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto"):
     if max_chunks == "least":
         max_chunks = 2 * len(small)
     ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], dev(small), dev(big), H,
-                             case["kp"].shape[3] ** -0.5, window, None, max_chunks, min_tiles)
+                             case["kp"].shape[3] ** -0.5, window, None, max_chunks, min_tiles, max_rows)
     return out, len(small), len(big)
 
 
@@ -602,6 +602,30 @@ def test_paged_attention_mfma_long_context(ops, cut, longest):
     seqs = [(longest, 1), (3000, 200), (70, 1)]
     case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=24, poison=True)
     out, _, _ = _run_mfma(ops, case, seqs, H, KV, 0, cut)
+    assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("n_items", [24, 64, 300])
+@pytest.mark.parametrize("cut", ["coarse", "fine"])
+def test_paged_attention_mfma_many_decoding_sequences(ops, n_items, cut):
+    """A decode step of dozens and hundreds of sequences of very different lengths, one token
+    each, at Llama-3.1-8B's attention shape: the chunk list is long, items have from one chunk to
+    dozens, and the partial results are merged by the combine kernel that takes a workgroup a row
+    (few chunks: 24 and 64 sequences cut coarsely) or by the one that takes a workgroup a kv head."""
+    import numpy as np
+
+    H, KV, hd, P = 32, 8, 128, 64
+    rng = np.random.default_rng(n_items)
+    lens = rng.integers(0, 2500 if n_items < 100 else 700, n_items)
+    lens[0], lens[1], lens[2] = 0, 63, 4000  # a first token, the last of a tile, one far longer than the rest
+    seqs = [(int(n), 1) for n in lens]
+    case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=25)
+    max_chunks = 2 * n_items if cut == "coarse" else 4096
+    by_rows = max_chunks * KV * (H // KV) <= 8192  # COMBINE_ROWS_MAX_GROUPS in attention_mfma.hip
+    assert by_rows == (cut == "coarse" and n_items <= 64)
+    out, n_small, n_big = _run_mfma(ops, case, seqs, H, KV, 0, cut, max_rows=H // KV)  # as a decode step has it
+    assert n_small == n_items and not n_big
+    assert torch.isfinite(out).all()
     assert torch.allclose(out.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
 
 

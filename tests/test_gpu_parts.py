@@ -160,7 +160,8 @@ class _HybridArch:
             else:
                 mixer = PartSpec(l["mixer"], f"{p}.mix", dict(dim=D, decay=l["decay"]))
             ffn = PartSpec(l.get("ffn", "swiglu"), f"{p}.ffn", dict(dim=D, hidden_dim=l["F"], **l.get("ffn_options", {})))
-            layers.append(LayerSpec(mixer, ffn, norm(f"{p}.n1"), norm(f"{p}.n2")))
+            layers.append(LayerSpec(mixer, ffn, norm(f"{p}.n1"), norm(f"{p}.n2"), l.get("arrangement", "pre_norm"),
+                                    {name: norm(f"{p}.{name}") for name in l.get("extra_norms", ())}))
         order = tuple(RunEntry(o[0], o[1]) for o in a["order"])
         return ModelLayout(D, a["vocab"], PartSpec("embedding", "emb", dict(vocab_size=a["vocab"], dim=D)),
                            tuple(layers), order, norm("final"),
@@ -201,13 +202,17 @@ def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32, ffns=None, position
             m = plain_attention(q, k, v, l.get("window")).reshape(T, H * hd) @ w[f"{p}.attn.o_proj.weight"].T
         else:
             m = mixers[l["mixer"]](x, w, p, l)
+        sandwich = l.get("arrangement") == "toy_sandwich"  # a norm after the mixer and after the feed-forward too
+        if sandwich:
+            m = plain_rmsnorm(m, w[f"{p}.post_mixer.weight"], a["eps"])
         h = h + m
         x = plain_rmsnorm(h, w[f"{p}.n2.weight"], a["eps"])
         if l.get("ffn", "swiglu") != "swiglu":
             h = h + ffns[l["ffn"]](x, w, p, l)
             continue
-        h = h + plain_swiglu(x, w[f"{p}.ffn.gate_proj.weight"], w[f"{p}.ffn.up_proj.weight"],
-                             w[f"{p}.ffn.down_proj.weight"])
+        f = plain_swiglu(x, w[f"{p}.ffn.gate_proj.weight"], w[f"{p}.ffn.up_proj.weight"],
+                         w[f"{p}.ffn.down_proj.weight"])
+        h = h + (plain_rmsnorm(f, w[f"{p}.post_ffn.weight"], a["eps"]) if sandwich else f)
     return (plain_rmsnorm(h, w["final.weight"], a["eps"]) @ w["head.weight"].T).float()
 
 
@@ -282,6 +287,13 @@ def _register_toy():
             return StateNeed((self.dim,), torch.float32)
 
         def forward(self, x, ctx, store):
+            if int(ctx.q_lens.max()) == 1:
+                # one token a sequence (the steps that are recorded and replayed): everything that changes
+                # from step to step comes from the context's device tensors
+                rows = ctx.slot_ids.long()
+                s = store.state.index_select(0, rows) * self.decay + x.float()
+                store.state.index_copy_(0, rows, s)
+                return (s @ self.w.float().T).to(x.dtype)
             out = torch.empty_like(x)
             at = 0
             for b in range(ctx.n_seqs):
@@ -318,7 +330,7 @@ def test_toy_mixer_with_state_of_its_own(tmp_path, hybrid_arch):
         model = Model.from_folder(folder, torch.float32, DEV)
         assert sorted(model.state_needs()) == [0, 2]
         runner = ModelRunner(model, page_size=16, max_tokens=256, max_requests=2)
-        assert len(runner.groups) == 1 and runner.storage.state[0].shape == (2, 48)
+        assert len(runner.groups) == 1 and runner.storage.state[0].shape == (2 + 1, 48)  # and a row that is nobody's
         lengths = {"a": 37, "b": 20, "c": 9}
         g = torch.Generator().manual_seed(5)
         toks = {r: torch.randint(0, 97, (n,), generator=g).tolist() for r, n in lengths.items()}
@@ -327,6 +339,19 @@ def test_toy_mixer_with_state_of_its_own(tmp_path, hybrid_arch):
         got = run_trace(runner, traces.mixed(lengths, max_live=2, seed=1), toks)
         assert_close(got, want, torch.float32, None, "toy")
         assert runner.cache.free_slots() == 2
+        # state of fixed size does not keep a model from recorded decode steps: three requests decode
+        # together from a step recorded for four (the stand-in's state is a row of nobody's), the
+        # warm-up before the recording leaves every request's state as it was
+        runner = ModelRunner(model, page_size=16, max_tokens=256, max_requests=3)
+        runner.graph_capacity = lambda n: 4 if n > 1 else 1
+        assert runner.use_graphs
+        n_head = {"a": 12, "b": 5, "c": 1}
+        trace = [([(r, 0, n)], []) for r, n in n_head.items()]
+        trace += [([(r, n_head[r] + s, 1) for r in n_head], []) for s in range(8)]
+        trace += [([("a", 20 + s, 1)], []) for s in range(17)]  # a alone: another recorded step
+        got = run_trace(runner, trace, toks)
+        assert sorted(c for c, _ in runner.graphs) == [1, 4]
+        assert_close(got, {"a": want["a"], "b": want["b"][:13], "c": want["c"]}, torch.float32, None, "toy, recorded")
     finally:
         unregister_part("mixer", "toy_ema")
 
@@ -436,3 +461,48 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, hybrid_arch
         unregister_part("feed_forward", "toy_routed")
         unregister_part("position", "toy_linear")
 
+
+
+# ------------------------------------------------- an arrangement with four norms
+def test_toy_arrangement_with_norms_of_its_own(tmp_path, hybrid_arch):
+    """A layer may own more norms than the two before its mixer and its feed-forward: a toy
+    arrangement, registered here, norms each part's output as well before it joins the residual
+    stream.  The layout names the further norms; the builder hands them over by name; their
+    tensors are loaded and checked like any other part's."""
+    from fastgen_amd.engine import Model, ModelRunner
+    from fastgen_amd.parts import register_part, unregister_part
+
+    class Sandwich:
+        def __init__(self, mixer, ffn, mixer_norm, ffn_norm, extra):
+            self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+            self.post_mixer, self.post_ffn = extra["post_mixer"], extra["post_ffn"]
+
+        def forward(self, h, pending, ctx, store):
+            x = self.mixer_norm.forward(h, pending, ctx.act_dtype)
+            mixed = self.mixer.forward(x, ctx, store)
+            mixed = self.post_mixer.forward(torch.zeros_like(h), mixed, ctx.act_dtype)  # the norm of 0 + mixed
+            x = self.ffn_norm.forward(h, mixed, ctx.act_dtype)
+            return self.post_ffn.forward(torch.zeros_like(h), self.ffn.forward(x), ctx.act_dtype)
+
+    register_part("arrangement", "toy_sandwich", lambda spec, *parts: Sandwich(*parts), replace=True)
+    try:
+        four = dict(arrangement="toy_sandwich", extra_norms=("post_mixer", "post_ffn"))
+        args = dict(dim=64, vocab=101, eps=1e-5, theta=1000.0, layers=[
+            dict(mixer="attention", H=4, KV=2, hd=16, F=72, **four),
+            dict(mixer="attention", H=2, KV=1, hd=32, F=96),  # and a plain pre-norm layer beside it
+            dict(mixer="attention", H=4, KV=4, hd=16, F=40, **four),
+        ], order=[(0, None), (1, None), (2, None)])
+        folder, w = _hybrid_case(tmp_path, args)
+        assert "blocks.0.post_mixer.weight" in w and "blocks.1.post_mixer.weight" not in w
+        lengths = {"a": 50, "b": 21, "c": 3}
+        g = torch.Generator().manual_seed(6)
+        toks = {r: torch.randint(0, 101, (n,), generator=g).tolist() for r, n in lengths.items()}
+        want = {r: _plain_hybrid(w, args, t, {}) for r, t in toks.items()}
+        noise = {r: _plain_hybrid(w, args, t, {}, torch.bfloat16) for r, t in toks.items()}
+        for dtype in (torch.float32, torch.bfloat16):
+            model = Model.from_folder(folder, dtype, DEV)
+            runner = ModelRunner(model, page_size=16, max_tokens=256, max_requests=3)
+            for tr in (traces.whole(lengths), traces.tail(lengths, 8), traces.mixed(lengths, max_live=3, seed=4)):
+                assert_close(run_trace(runner, tr, toks), want, dtype, noise, "sandwich")
+    finally:
+        unregister_part("arrangement", "toy_sandwich")
