@@ -23,6 +23,93 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define EPI_STORE 0
 #define EPI_SILU_MUL 1
 #define EPI_ROPE_KV 2  // w = [q; k; v] projections: rotate q and k, q to y, k and v into their cache pages
+#define EPI_RESIDUAL 3  // the product is added to the fp32 residual stream; see Residual
+
+// For at most 16 rows the two RMSNorms of a layer need no kernels of their own.  The product that
+// feeds the residual stream (EPI_RESIDUAL) adds its result to h, stores h * norm_w (not yet divided by
+// the row's root mean square) as the next product's x, and one sum of squares of h per row and
+// workgroup.  The next product (RowScale) adds those sums up, in a fixed order, and multiplies its
+// result rows by rsqrt(mean + eps): W (x' * r) = r * (W x').  x' is rounded to bfloat16 as the normed
+// row would be, to the same relative error.
+struct RowScale {
+  const float* ssq;  // [M, n_parts] sums of squares whose sum over n_parts is the row's; null: rows are taken as they are
+  int n_parts;
+  float inv_dim, eps;
+};
+struct Residual {
+  float* h;             // [M, N] fp32 residual stream, updated in place
+  int ldh;
+  const void* norm_w;   // [N] weight of the norm that follows
+  int norm_w_f32;       // its dtype: fp32 or bf16
+  bf16_t* x_out;        // [M, N] h * norm_w
+  int ldxo;
+  float* ssq_out;       // [M, gridDim.x]
+};
+
+// The sum of a row's partial sums of squares is taken by 1/16 of the workgroup's threads: each adds up
+// a strided share early (eight loads in flight at a time, issued before the product's own, so that
+// their latency passes during the product), the shares are added in the end.
+template <int THREADS>
+__device__ __forceinline__ float row_scale_begin(const RowScale& sc, int M) {
+  constexpr int TPR = THREADS / 16;
+  const int m = min((int)threadIdx.x / TPR, M - 1), sub = threadIdx.x % TPR;
+  float s = 0.f;
+  if (sc.ssq) {  // uniform
+    const float* row = sc.ssq + (size_t)m * sc.n_parts;
+    for (int p0 = 0; p0 < sc.n_parts; p0 += 8 * TPR) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = row[min(p0 + sub + j * TPR, sc.n_parts - 1)];  // never conditional
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += p0 + sub + j * TPR < sc.n_parts ? v[j] : 0.f;
+    }
+  }
+  return s;
+}
+template <int THREADS>
+__device__ __forceinline__ void row_scale_end(const RowScale& sc, float part, float* rscale /* LDS [16] */) {
+  constexpr int TPR = THREADS / 16;  // 16 or 32: the threads of a row are neighbours in one wave
+#pragma unroll
+  for (int w = TPR / 2; w > 0; w >>= 1) part += __shfl_xor(part, w, FG_WAVE);
+  if (threadIdx.x % TPR == 0) rscale[threadIdx.x / TPR] = sc.ssq ? rsqrtf(part * sc.inv_dim + sc.eps) : 1.f;
+}
+
+// EPI_RESIDUAL for one 16 x 16 tile whose waves' partial sums lie in red[WAVES][256] (row m, column c at
+// m * 16 + c): the first 256 threads take an element each.  What they need from memory (h and the
+// norm's weight at their element) is asked for before the product (residual_begin), so that the
+// epilogue does not wait for it.
+struct ResidualRegs { float h, w; };
+__device__ __forceinline__ ResidualRegs residual_begin(const Residual& rs, int n0, int M, int N) {
+  ResidualRegs r{0.f, 0.f};
+  const int e = threadIdx.x;
+  if (e < 256) {  // whole waves
+    const int m = min(e >> 4, M - 1), n = min(n0 + (e & 15), N - 1);
+    r.h = rs.h[(size_t)m * rs.ldh + n];
+    r.w = rs.norm_w_f32 ? ((const float*)rs.norm_w)[n] : (float)((const bf16_t*)rs.norm_w)[n];
+  }
+  return r;
+}
+template <int WAVES>
+__device__ __forceinline__ void residual_epilogue(const float (*red)[256], const float* rscale, const Residual& rs,
+                                                  const ResidualRegs& pre, int n0, int M, int N) {
+  const int e = threadIdx.x;
+  if (e >= 256) return;  // (whole waves)
+  const int m = e >> 4, c = e & 15, n = n0 + c;
+  float s = 0.f;
+#pragma unroll
+  for (int wv = 0; wv < WAVES; ++wv) s += red[wv][e];
+  float sq = 0.f;
+  if (m < M && n < N) {
+    const float hv = pre.h + s * rscale[m];
+    rs.h[(size_t)m * rs.ldh + n] = hv;
+    rs.x_out[(size_t)m * rs.ldxo + n] = (bf16_t)(hv * pre.w);
+    sq = hv * hv;
+  }
+  // the 16 columns of a row are 16 neighbouring lanes
+#pragma unroll
+  for (int w = 8; w > 0; w >>= 1) sq += __shfl_xor(sq, w, FG_WAVE);
+  if (c == 0 && m < M) rs.ssq_out[(size_t)m * gridDim.x + blockIdx.x] = sq;
+}
 
 // What the EPI_ROPE_KV epilogue needs beside the product (rope_kv.hip does the same as a kernel of
 // its own for steps with more rows).
@@ -44,9 +131,14 @@ __device__ __forceinline__ bf16x8 gs_zero8() {
 template <int MB, int WAVES, int EPI, class TY>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
-    int ldy, int M, int N, int K) {
+    int ldy, int M, int N, int K, RowScale sc, Residual rs) {
   constexpr int U = MB <= 2 ? 8 : 4;  // k steps in flight
   __shared__ float red[WAVES][MB * 256];
+  __shared__ float rscale[16];
+  static_assert(EPI != EPI_RESIDUAL || MB == 1, "the residual epilogue is for at most 16 rows");
+  const float sc_part = MB == 1 ? row_scale_begin<WAVES * 64>(sc, M) : 0.f;
+  ResidualRegs pre{0.f, 0.f};
+  if (EPI == EPI_RESIDUAL) pre = residual_begin(rs, blockIdx.x * 16, M, N);
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
@@ -84,13 +176,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   // acc[mb][i] = C[n = 4g + i][m = 16 mb + r16]
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) *(f32x4*)(&red[wave][(mb * 16 + r16) * 16 + 4 * g]) = acc[mb];
+  if (MB == 1) row_scale_end<WAVES * 64>(sc, sc_part, rscale);
   __syncthreads();
-  if (EPI == EPI_STORE) {
+  if (EPI == EPI_RESIDUAL) {
+    if constexpr (MB == 1) residual_epilogue<WAVES>(red, rscale, rs, pre, n0, M, N);
+  } else if (EPI == EPI_STORE) {
     for (int e = threadIdx.x; e < MB * 256; e += WAVES * 64) {
       float s = 0.f;
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) s += red[wv][e];
       const int m = e >> 4, n = n0 + (e & 15);
+      if (MB == 1) s *= rscale[m];
       if (m < M && n < N) y[(size_t)m * ldy + n] = from_f<TY>(s);
     }
   } else {
@@ -102,6 +198,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
       for (int wv = 0; wv < WAVES; ++wv) {
         gate += red[wv][m * 16 + j];
         up += red[wv][m * 16 + 8 + j];
+      }
+      if (MB == 1) {
+        gate *= rscale[m];
+        up *= rscale[m];
       }
       const int col = n0 / 2 + j;
       if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + col] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
@@ -120,9 +220,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 template <int WAVES, int EPI, class TY>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
-    int ldy, int M, int N, int K, RopeKv rk) {
+    int ldy, int M, int N, int K, RopeKv rk, RowScale sc, Residual rs) {
   constexpr int U = 8;
   __shared__ float red[WAVES][256];
+  __shared__ float rscale[16];
+  const float sc_part = row_scale_begin<WAVES * 64>(sc, M);
+  ResidualRegs pre{0.f, 0.f};
+  if (EPI == EPI_RESIDUAL) pre = residual_begin(rs, blockIdx.x * 16, M, N);
   __shared__ __attribute__((aligned(16))) bf16_t xs[WAVES][4 * U * 16 * 8];  // [k chunk][row][8]
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
@@ -165,8 +269,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     }
   }
   *(f32x4*)(&red[wave][r16 * 16 + 4 * g]) = acc;
+  row_scale_end<WAVES * 64>(sc, sc_part, rscale);
   __syncthreads();
-  if (EPI == EPI_ROPE_KV) {
+  if (EPI == EPI_RESIDUAL) {
+    residual_epilogue<WAVES>(red, rscale, rs, pre, n0, M, N);
+  } else if (EPI == EPI_ROPE_KV) {
     // 16 columns = 8 pairs of one head of q, k or v (head sizes are multiples of 16)
     for (int e = threadIdx.x; e < 128; e += WAVES * 64) {
       const int m = e >> 3, p = e & 7, n = n0 + 2 * p;
@@ -177,6 +284,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
         a += red[wv][m * 16 + 2 * p];
         b += red[wv][m * 16 + 2 * p + 1];
       }
+      a *= rscale[m];
+      b *= rscale[m];
       const int q_cols = rk.n_heads * rk.hd, k_cols = rk.n_kv * rk.hd;
       const int d = n % rk.hd;
       if (n < q_cols + k_cols && rk.table && d < rk.rotary_dim) {
@@ -214,6 +323,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) s += red[wv][e];
       const int m = e >> 4, n = n0 + (e & 15);
+      s *= rscale[m];
       if (m < M && n < N) y[(size_t)m * ldy + n] = from_f<TY>(s);
     }
   } else {
@@ -225,6 +335,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
         gate += red[wv][m * 16 + j];
         up += red[wv][m * 16 + 8 + j];
       }
+      gate *= rscale[m];
+      up *= rscale[m];
       if (m < M && n0 + 8 + j < N) y[(size_t)m * ldy + n0 / 2 + j] = from_f<TY>(gate / (1.f + __expf(-gate)) * up);
     }
   }
@@ -318,24 +430,24 @@ __global__ __launch_bounds__(256, U == 4 ? 4 : 2) void gemm_skinny64_kernel(
 
 template <int MB, int EPI, class TY>
 static void launch_skinny(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
-                          int K, hipStream_t stream) {
+                          int K, const RowScale& sc, const Residual& rs, hipStream_t stream) {
   const int blocks = (N + 15) / 16;
   if (MB == 1 && M > 1) {  // one row of x is a broadcast already
     if (blocks >= 1024)
       gemm_skinny16_kernel<4, EPI, TY><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K, RopeKv{});
+                                                                   (TY*)y, ldy, M, N, K, RopeKv{}, sc, rs);
     else
       gemm_skinny16_kernel<8, EPI, TY><<<blocks, 512, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K, RopeKv{});
+                                                                   (TY*)y, ldy, M, N, K, RopeKv{}, sc, rs);
     return;
   }
   // few blocks: more waves a block, so that enough loads are in flight on every CU
   if (blocks >= 1024)
     gemm_skinny_kernel<MB, 4, EPI, TY><<<blocks, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K);
+                                                                   (TY*)y, ldy, M, N, K, sc, rs);
   else
     gemm_skinny_kernel<MB, 8, EPI, TY><<<blocks, 512, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, ldw,
-                                                                   (TY*)y, ldy, M, N, K);
+                                                                   (TY*)y, ldy, M, N, K, sc, rs);
 }
 
 // x [M, K] bf16 (M <= 64), w [N, K] bf16, K % 8 == 0, rows 16-byte aligned.
@@ -349,14 +461,16 @@ extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, vo
   if (epilogue == EPI_STORE && ldy < N) return FG_ERR_ARG;
   if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
   const int mb = (M + 15) / 16;
+  const RowScale sc{nullptr, 0, 0.f, 0.f};
+  const Residual rs{};
 #define GO(MB)                                                                                        \
   do {                                                                                                \
     if (epilogue == EPI_STORE && out_dtype == FG_BF16)                                                \
-      launch_skinny<MB, EPI_STORE, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, stream);                  \
+      launch_skinny<MB, EPI_STORE, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);          \
     else if (epilogue == EPI_STORE && out_dtype == FG_F32)                                            \
-      launch_skinny<MB, EPI_STORE, float>(x, ldx, w, ldw, y, ldy, M, N, K, stream);                   \
+      launch_skinny<MB, EPI_STORE, float>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);           \
     else if (epilogue == EPI_SILU_MUL && out_dtype == FG_BF16)                                        \
-      launch_skinny<MB, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, stream);               \
+      launch_skinny<MB, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);       \
     else                                                                                              \
       return FG_ERR_ARG;                                                                              \
   } while (0)
@@ -365,6 +479,32 @@ extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, vo
   else if (mb == 3) GO(3);
   else GO(4);
 #undef GO
+  return fg_launch_status();
+}
+
+// The same for at most 16 rows with the layer's norms folded into the products (see RowScale and
+// Residual above).  ssq [M, n_parts] (null: x is taken as it is), dim = the width that the sums of
+// squares run over.  epilogue 0 and 1 as above (y bf16); epilogue 3: y is not written; h [M, N] fp32
+// += the product, x_out [M, N] bf16 = h * norm_w, ssq_out [M, ceil(N / 16)] = the sums of squares of
+// h over each workgroup's 16 columns.
+extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
+                                    int K, int epilogue, const float* ssq, int n_parts, int dim, float eps,
+                                    float* h, int ldh, const void* norm_w, int norm_w_dtype, void* x_out, int ldxo,
+                                    float* ssq_out, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return FG_OK;
+  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return FG_ERR_ARG;
+  if (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))) return FG_ERR_ARG;
+  if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || !y)) return FG_ERR_ARG;
+  if (epilogue == EPI_STORE && (ldy < N || !y)) return FG_ERR_ARG;
+  if (epilogue == EPI_RESIDUAL && (!h || !norm_w || !x_out || !ssq_out || ldh < N || ldxo < N ||
+                                   (norm_w_dtype != FG_F32 && norm_w_dtype != FG_BF16)))
+    return FG_ERR_ARG;
+  const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
+  const Residual rs{h, ldh, norm_w, norm_w_dtype == FG_F32, (bf16_t*)x_out, ldxo, ssq_out};
+  if (epilogue == EPI_STORE) launch_skinny<1, EPI_STORE, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
+  else if (epilogue == EPI_SILU_MUL) launch_skinny<1, EPI_SILU_MUL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
+  else if (epilogue == EPI_RESIDUAL) launch_skinny<1, EPI_RESIDUAL, bf16_t>(x, ldx, w, ldw, y, ldy, M, N, K, sc, rs, stream);
+  else return FG_ERR_ARG;
   return fg_launch_status();
 }
 
@@ -405,24 +545,28 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
 // q, k, v projections of at most 16 rows with the rotation and the cache write in the epilogue:
 // w = [q rows; k rows; v rows] ([(H + 2 KV) * hd, K]); y = rotated q [M, H * hd]; rotated k and v go
 // to slots[m] of the pages.  table: cos/sin of the rows' positions (null: no rotation).
+// ssq [M, n_parts] (null: x is taken as it is): the rows' sums of squares for the norm folded into this product.
 extern "C" int fg_gemm_skinny_qkv(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int K,
                                   const float* table, const int* slots, void* k_pages, void* v_pages,
                                   int n_heads, int n_kv, int hd, int rotary_dim, int page_size,
-                                  hipStream_t stream) {
+                                  const float* ssq, int n_parts, int dim, float eps, hipStream_t stream) {
   if (M <= 0) return FG_OK;
   const int N = (n_heads + 2 * n_kv) * hd;
   if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || hd % 16 || n_heads <= 0 ||
       n_kv <= 0 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 || page_size <= 0 || page_size % 8 ||
-      ldy < n_heads * hd || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table))
+      ldy < n_heads * hd || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table) ||
+      (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))))
     return FG_ERR_ARG;
+  const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
+  const Residual rs{};
   const RopeKv rk{rotary_dim ? table : nullptr, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
                   n_heads, n_kv, hd, rotary_dim, page_size};
   const int blocks = N / 16;
   if (blocks >= 1024)
     gemm_skinny16_kernel<4, EPI_ROPE_KV, bf16_t><<<blocks, 256, 0, stream>>>(
-        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk);
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk, sc, rs);
   else
     gemm_skinny16_kernel<8, EPI_ROPE_KV, bf16_t><<<blocks, 512, 0, stream>>>(
-        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk);
+        (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (bf16_t*)y, ldy, M, N, K, rk, sc, rs);
   return fg_launch_status();
 }

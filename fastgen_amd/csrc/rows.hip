@@ -227,6 +227,37 @@ extern "C" int fg_rmsnorm(const void* x, const void* w, void* out, int n_rows, i
   return fg_launch_status();
 }
 
+// Rows times rsqrt(sum of the row's partial sums of squares / dim + eps): the second half of a norm
+// whose first half (the weight, the sums of squares) was done where the rows were made.
+template <class TA>
+__global__ __launch_bounds__(ROWS_THREADS) void scale_rows_kernel(
+    const TA* __restrict__ x, const float* __restrict__ ssq, TA* __restrict__ out, int width, int n_parts,
+    float inv_dim, float eps) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  float ss = 0.f;
+  for (int p = threadIdx.x; p < n_parts; p += ROWS_THREADS) ss += ssq[(size_t)r * n_parts + p];
+  ss = block_sum(ss, red);
+  const float rstd = rsqrtf(ss * inv_dim + eps);
+  for (int i = threadIdx.x; i < width; i += ROWS_THREADS)
+    out[(size_t)r * width + i] = from_f<TA>(to_f<TA>(x[(size_t)r * width + i]) * rstd);
+}
+
+extern "C" int fg_scale_rows(const void* x, const float* ssq, void* out, int n_rows, int width, int n_parts,
+                             int dim, float eps, int act_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return FG_OK;
+  if (width <= 0 || n_parts <= 0 || dim <= 0 || !(eps >= 0.f)) return FG_ERR_ARG;
+  if (act_dtype == FG_F32)
+    scale_rows_kernel<float><<<n_rows, ROWS_THREADS, 0, stream>>>((const float*)x, ssq, (float*)out, width, n_parts,
+                                                                  1.f / (float)dim, eps);
+  else if (act_dtype == FG_BF16)
+    scale_rows_kernel<bf16_t><<<n_rows, ROWS_THREADS, 0, stream>>>((const bf16_t*)x, ssq, (bf16_t*)out, width,
+                                                                   n_parts, 1.f / (float)dim, eps);
+  else
+    return FG_ERR_ARG;
+  return fg_launch_status();
+}
+
 // ------------------------------------------------------------- SiLU(g) * u
 // gu is [n_rows, 2*hidden] with gate and up columns interleaved in groups of
 // 8: columns 16k .. 16k+7 are gate 8k .. 8k+7, columns 16k+8 .. 16k+15 their up

@@ -15,6 +15,7 @@ from typing import Any, Dict, List, Mapping, Optional, Sequence
 import torch
 
 from ..config import ModelLayout, PartSpec, get_architecture, read_config_json
+from ..kernels.ops import ScaledRows
 from ..parts import LayerStore, PagedNeed, StateNeed, TensorSpec, build_part
 from ..weights.source import RandomSource, SafetensorsSource, TensorSource, check_against_specs
 from .context import StepContext
@@ -137,9 +138,19 @@ class Model:
         if not self.loaded:
             raise RuntimeError("the model has no weights yet")
         h = self.parts.embed.forward(ctx.tokens)
-        pending: Optional[torch.Tensor] = None
-        for i, entry in enumerate(self.layout.order):
-            pending = self.parts.blocks[entry.layer].forward(h, pending, ctx, stores[i])
+        pending = None  # rows still to be added to h, or ScaledRows (added already, the next norm half done)
+        blocks, order = self.parts.blocks, self.layout.order
+        for i, entry in enumerate(order):
+            block = blocks[entry.layer]
+            if getattr(block, "folds_norms", False):
+                # the norm that follows this block is the next block's first, if that block can take over
+                after = blocks[order[i + 1].layer] if i + 1 < len(order) else None
+                next_norm = after.mixer_norm if getattr(after, "folds_norms", False) else None
+                pending = block.forward(h, pending, ctx, stores[i], next_norm=next_norm)
+            else:
+                pending = block.forward(h, None if isinstance(pending, ScaledRows) else pending, ctx, stores[i])
+        if isinstance(pending, ScaledRows):
+            pending = None  # h holds the sum already
         if ctx.n_out == 0:
             return None
         x = self.parts.final_norm.forward(h, pending, ctx.act_dtype, rows=ctx.out_rows)

@@ -10,7 +10,7 @@ with fp32 accumulation; logits are asked for in fp32 directly.
 
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -63,11 +63,37 @@ def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
     return max(1, min(8, 512 // blocks, k // (1024 if rows > 48 else 512)))
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           partials_ok: bool = False) -> torch.Tensor:
+def fold_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Few rows of bfloat16: the norms around a product can be folded into the products
+    (:class:`~fastgen_amd.kernels.ops.ScaledRows`)."""
+    return skinny_ok(x, w)
+
+
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           partials_ok: bool = False, residual: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None):
     """``x @ w.T``.  With ``partials_ok`` the result may come as fp32 ``[S, M, N]``
     partial sums whose sum over ``S`` is the product (the caller hands it to a
-    norm, which adds them in order)."""
+    norm, which adds them in order).
+
+    ``x`` may be :class:`~fastgen_amd.kernels.ops.ScaledRows`.  ``residual`` = (h, norm weight,
+    eps) asks for more than the product: add it to the fp32 residual stream ``h`` and prepare the
+    RMSNorm that follows.  Where that can be folded into the product's kernel (few rows, bfloat16)
+    the result is ``ScaledRows`` and ``h`` is updated; where not, the plain product comes back and
+    adding and norming are the caller's."""
+    scaled = x if isinstance(x, ops.ScaledRows) else None
+    if scaled is not None:
+        if not fold_ok(scaled.rows, w):
+            x, scaled = scaled.materialize(), None
+        else:
+            x = scaled.rows
+    if residual is not None and x.is_cuda and fold_ok(x, w) and out_dtype in (None, torch.bfloat16):
+        h, norm_w, eps = residual
+        if h.dtype == torch.float32 and h.is_contiguous() and h.shape == (x.shape[0], w.shape[0]):
+            return ops.gemm_skinny_residual(scaled or x, w, h, norm_w, eps)
+    if scaled is not None:
+        if out_dtype in (None, torch.bfloat16):
+            return ops.gemm_skinny(scaled, w, torch.bfloat16, wide=False)
+        x = scaled.materialize()
     if not x.is_cuda:
         raise ops.KernelArgumentError("fastgen_amd runs on the GPU only; got a tensor on " + str(x.device))
     out_dtype = out_dtype or x.dtype

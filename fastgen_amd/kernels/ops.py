@@ -9,6 +9,7 @@ is not on a GPU is refused.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 import os
 from typing import Optional
 
@@ -458,16 +459,93 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+@dataclass
+class ScaledRows:
+    """Rows that are not yet divided by their root mean square: the true row ``t`` is
+    ``rows[t] * rsqrt(sum(ssq[t]) / dim + eps)``.  For few rows the norm before a matrix product
+    is folded into the products around it: the one before stores ``rows`` and the sums of squares
+    of its workgroups' columns (:func:`gemm_skinny_residual`), the one after scales its result
+    rows (``x @ w.T`` is linear in a row's scale)."""
+
+    rows: torch.Tensor  # [T, dim] bfloat16
+    ssq: torch.Tensor  # [T, n_parts] float32
+    dim: int
+    eps: float
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    def materialize(self) -> torch.Tensor:
+        """The rows themselves (a kernel of its own: for a consumer that does not take the pair)."""
+        return scale_rows(self.rows, self.ssq, self.dim, self.eps)
+
+
+def _row_scale_args(x, M: int):
+    """C arguments (ssq, n_parts, dim, eps) for ``x`` a tensor or :class:`ScaledRows`."""
+    if not isinstance(x, ScaledRows):
+        return ctypes.c_void_p(0), 0, 0, ctypes.c_float(0.0)
+    ssq = x.ssq
+    _need(ssq.dtype == torch.float32 and ssq.is_contiguous() and ssq.dim() == 2 and ssq.shape[0] == M
+          and ssq.is_cuda, "ssq must be contiguous float32 [M, n_parts] on the GPU")
+    _need(x.dim > 0 and x.eps >= 0, "ScaledRows needs dim > 0 and eps >= 0")
+    return _ptr(ssq), ssq.shape[1], int(x.dim), ctypes.c_float(x.eps)
+
+
+def scale_rows(rows: torch.Tensor, ssq: torch.Tensor, dim: int, eps: float) -> torch.Tensor:
+    """``rows[t] * rsqrt(sum(ssq[t]) / dim + eps)`` in the dtype of ``rows``."""
+    _gpu(rows, ssq)
+    _need(rows.dim() == 2 and rows.is_contiguous() and ssq.dim() == 2 and ssq.is_contiguous()
+          and ssq.dtype == torch.float32 and ssq.shape[0] == rows.shape[0], "rows [T, D], ssq float32 [T, n_parts]")
+    out = torch.empty_like(rows)
+    st = _lib.load("rows").fg_scale_rows(_ptr(rows), _ptr(ssq), _ptr(out), rows.shape[0], rows.shape[1],
+                                         ssq.shape[1], int(dim), ctypes.c_float(eps), _code(rows), _stream(rows))
+    _check(st, "scale_rows")
+    return out
+
+
+def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, h: torch.Tensor, norm_weight: torch.Tensor,
+                         eps: float) -> ScaledRows:
+    """For at most 16 rows: ``h += x @ w.T`` on the fp32 residual stream ``h [M, N]`` and, in the same
+    kernel, what the RMSNorm that follows needs: ``h * norm_weight`` in bfloat16 and a sum of squares
+    of ``h`` per row and workgroup (16 columns).  ``x`` may itself be :class:`ScaledRows`."""
+    rows = x.rows if isinstance(x, ScaledRows) else x
+    _gpu(rows, w, h, norm_weight)
+    M, K = rows.shape
+    N = w.shape[0]
+    _need(rows.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] == K and 0 < M <= 16,
+          "gemm_skinny_residual takes bfloat16 x [M<=16, K] and w [N, K]")
+    _need(K % 8 == 0 and rows.stride(1) == 1 and w.stride(1) == 1 and rows.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+          and rows.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "K must be a multiple of 8, rows 16-byte aligned")
+    _need(h.dtype == torch.float32 and h.shape == (M, N) and h.stride(1) == 1, "h must be float32 [M, N]")
+    _need(norm_weight.shape == (N,) and norm_weight.is_contiguous()
+          and norm_weight.dtype in (torch.float32, torch.bfloat16), "norm_weight must be [N], float32 or bfloat16")
+    n_parts = -(-N // 16)
+    x_out = torch.empty((M, N), dtype=torch.bfloat16, device=rows.device)
+    ssq_out = torch.empty((M, n_parts), dtype=torch.float32, device=rows.device)
+    sc = _row_scale_args(x, M)
+    st = _lib.load("gemm_skinny").fg_gemm_skinny_fused(
+        _ptr(rows), rows.stride(0), _ptr(w), w.stride(0), ctypes.c_void_p(0), 0, M, N, K, 3, *sc,
+        _ptr(h), h.stride(0), _ptr(norm_weight), _code(norm_weight), _ptr(x_out), x_out.stride(0), _ptr(ssq_out),
+        _stream(rows))
+    _check(st, "gemm_skinny_residual")
+    return ScaledRows(x_out, ssq_out, N, float(eps))
+
+
+def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 silu_mul_epilogue: bool = False, k_splits: int = 1, wide: Optional[bool] = None) -> torch.Tensor:
     """``x @ w.T`` for at most 64 rows of bf16 ``x`` on the matrix cores, built to
-    stream ``w [N, K]`` once.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
+    stream ``w [N, K]`` once.  ``x`` may be :class:`ScaledRows` (at most 16 rows, bfloat16 out): the
+    result rows are scaled.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
     ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
     ``[M, N/2]``.  With ``k_splits > 1`` the k range is cut over workgroups and the
     result is fp32 ``[k_splits, M, N]`` partial sums (for few output columns,
     where one workgroup per 64 columns would leave most of the GPU idle).
     ``wide`` picks the kernel for 17..64 rows (64 columns a workgroup, x shared
     through LDS); default: by the number of rows."""
+    scaled = x if isinstance(x, ScaledRows) else None
+    if scaled is not None:
+        x = scaled.rows
     _gpu(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16 operands")
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
@@ -486,7 +564,13 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     cols = N // 2 if silu_mul_epilogue else N
     y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
     lib = _lib.load("gemm_skinny")
-    if wide:
+    if scaled is not None:
+        _need(M <= 16 and not wide and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
+        st = lib.fg_gemm_skinny_fused(
+            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, 1 if silu_mul_epilogue else 0,
+            *_row_scale_args(scaled, M), ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0,
+            ctypes.c_void_p(0), _stream(x))
+    elif wide:
         st = lib.fg_gemm_skinny64(
             _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
             K, _code(y), 1 if silu_mul_epilogue else 0, _stream(x))
@@ -498,12 +582,15 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     return y
 
 
-def gemm_skinny_qkv(x: torch.Tensor, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots: torch.Tensor,
+def gemm_skinny_qkv(x, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots: torch.Tensor,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                     rotary_dim: int) -> torch.Tensor:
     """The q, k, v projections of at most 16 rows with :func:`rope_kv_write` in
     the product's epilogue: returns the rotated queries ``[M, H*hd]``; the rotated
-    keys and the values go straight into their cache pages."""
+    keys and the values go straight into their cache pages.  ``x`` may be :class:`ScaledRows`."""
+    scaled = x if isinstance(x, ScaledRows) else None
+    if scaled is not None:
+        x = scaled.rows
     _gpu(x, wqkv, table, slots, k_pages, v_pages)
     _need(x.dim() == 2 and wqkv.dim() == 2 and k_pages.dim() == 4, "x [M, K], wqkv [N, K], k_pages [n, KV, P, hd]")
     M, K = x.shape
@@ -525,7 +612,7 @@ def gemm_skinny_qkv(x: torch.Tensor, wqkv: torch.Tensor, table: Optional[torch.T
     st = _lib.load("gemm_skinny").fg_gemm_skinny_qkv(
         _ptr(x), x.stride(0), _ptr(wqkv), wqkv.stride(0), _ptr(q), q.stride(0), M, K,
         _ptr(table if rotary_dim else None), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_heads, n_kv, head_dim,
-        rotary_dim, page_size, _stream(x))
+        rotary_dim, page_size, *_row_scale_args(scaled, M), _stream(x))
     _check(st, "gemm_skinny_qkv")
     return q
 

@@ -18,6 +18,8 @@ from .base import LayerStore, Mixer, PagedNeed, TensorSpec, build_part, place, r
 
 
 class Attention(Mixer):
+    folds_norms = True  # takes ScaledRows and the ``then`` request (see parts.block)
+
     def __init__(self, spec) -> None:
         super().__init__(spec)
         o = spec.options
@@ -59,7 +61,10 @@ class Attention(Mixer):
     def paged_need(self) -> PagedNeed:
         return PagedNeed(self.n_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x: torch.Tensor, ctx: Any, store: LayerStore) -> torch.Tensor:
+    def forward(self, x, ctx: Any, store: LayerStore, then=None):
+        """``x``: the normed rows, or ``ScaledRows`` (a norm not yet finished, which the q/k/v product
+        finishes).  ``then``: a norm's ``fold_request``; the output projection may fold the addition
+        to the residual stream and that norm into its kernel and return ``ScaledRows``."""
         group = ctx.groups[store.group]
         q_width = self.n_heads * self.head_dim
         table = None
@@ -70,7 +75,10 @@ class Attention(Mixer):
             table = ctx.scratch.get(key)
             if table is None:
                 table = ctx.scratch[key] = ops.rope_table(ctx.positions, self.freqs)
-        if store.owns and self.head_dim % 16 == 0 and skinny_ok(x, self.wqkv):
+        rows = x.rows if isinstance(x, ops.ScaledRows) else x
+        if not (store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv)) and rows is not x:
+            x = x.materialize()
+        if store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv):
             # few rows (decode): rotation and cache write happen where the product is stored
             qkv = ops.gemm_skinny_qkv(x, self.wqkv, table, group.slots, store.k_pages, store.v_pages, self.n_heads,
                                       self.n_kv_heads, self.head_dim, self.position.rotary_dim)
@@ -82,10 +90,10 @@ class Attention(Mixer):
                 self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,
                 table=table,
             )
-        out = torch.empty((x.shape[0], q_width), dtype=x.dtype, device=x.device)
+        out = torch.empty((rows.shape[0], q_width), dtype=rows.dtype, device=rows.device)
         ops.paged_attention(qkv, out, store.k_pages, store.v_pages, group, ctx, self.n_heads, self.scale,
                             self.window or 0)
-        return linear(out, self.wo, partials_ok=True)
+        return linear(out, self.wo, partials_ok=True, residual=then)
 
 
 register_part("mixer", "attention", Attention)

@@ -11,11 +11,13 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear, wide_ok
+from ..kernels.linear import linear, skinny_ok, wide_ok
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
 class SwiGLU(FeedForward):
+    folds_norms = True  # takes ScaledRows and the ``then`` request (see parts.block)
+
     def __init__(self, spec) -> None:
         super().__init__(spec)
         self.dim = int(spec.options["dim"])
@@ -43,12 +45,17 @@ class SwiGLU(FeedForward):
         self.w_gate_up = place(ops.interleave_gate_up(gate, up), MATRIX, dtype, device)
         self.w_down = place(down, MATRIX, dtype, device)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if wide_ok(x, self.w_gate_up):
+    def forward(self, x, then=None):
+        """``x``: the normed rows, or ``ScaledRows`` (the gate/up product finishes the norm).  ``then``:
+        a norm's ``fold_request`` for the down projection (see ``Attention.forward``)."""
+        rows = x.rows if isinstance(x, ops.ScaledRows) else x
+        if rows is not x and not skinny_ok(rows, self.w_gate_up):
+            x = rows = x.materialize()
+        if wide_ok(rows, self.w_gate_up):
             act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True)
         else:
             act = ops.silu_mul(linear(x, self.w_gate_up))
-        return linear(act, self.w_down, partials_ok=True)
+        return linear(act, self.w_down, partials_ok=True, residual=then)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

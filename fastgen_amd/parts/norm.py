@@ -25,6 +25,11 @@ class RMSNorm(Norm):
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
         self.weight = place(tensors[self._name("weight")], VECTOR, dtype, device)
 
+    def fold_request(self, h: torch.Tensor):
+        """(h, weight, eps): what a matrix product needs to fold the addition to the residual stream
+        and this norm into its kernel (``fastgen_amd.kernels.linear.linear(residual=...)``)."""
+        return (h, self.weight, self.eps)
+
     def forward(self, h, delta, dtype, rows=None):
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=dtype, device=h.device)

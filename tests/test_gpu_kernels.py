@@ -412,6 +412,81 @@ def test_gemm_skinny_gate_up_epilogue(ops, M, F, K):
     assert (got - want).abs().max() <= 1e-2 * want.abs().max() + 1e-3
 
 
+@pytest.mark.parametrize("M", [1, 2, 8, 16])
+@pytest.mark.parametrize("N,K,F", [(240, 328, 200), (4096, 14336, 1000), (104, 64, 24), (520, 240, 328)])
+@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
+def test_norms_folded_into_the_products(ops, M, N, K, F, w_dtype):
+    """For few rows: ``h += x W^T`` with what the RMSNorm after it needs made in the same kernel
+    (h times the norm's weight, sums of squares per workgroup), and the products that take such
+    rows and scale their results: plain store, the gate/up product, and a second residual product;
+    each against the plain formulas ``h + x W^T`` and ``rmsnorm(h) W2^T``."""
+    torch.manual_seed(M + N)
+    eps = 1e-5
+    x = torch.randn(M, K).bfloat16()
+    w = (torch.randn(N, K) * K**-0.5).bfloat16()
+    h = torch.randn(M, N) * 3
+    nw = (1 + 0.2 * torch.randn(N)).to(w_dtype)
+    h_d = h.to(DEV)
+    sr = ops.gemm_skinny_residual(x.to(DEV), w.to(DEV), h_d, nw.to(DEV), eps)
+    h_new = h.double() + x.double() @ w.double().T
+    assert torch.allclose(h_d.cpu().double(), h_new, atol=1e-4 * float(h_new.abs().max()))
+    assert sr.rows.shape == (M, N) and sr.ssq.shape == (M, -(-N // 16)) and sr.dim == N
+    assert torch.allclose(sr.ssq.cpu().double().sum(1), (h_new * h_new).sum(1), rtol=1e-5)
+    normed = plain_rmsnorm(h_new.float(), nw.float(), eps)  # what the norm's own kernel would hand on
+    got = sr.materialize().cpu().float()
+    assert torch.allclose(got, normed, atol=2e-2 * float(normed.abs().max()), rtol=2e-2)
+    # consumers: a plain product, the gate/up product, a residual product on scaled rows
+    w2 = (torch.randn(F, N) * N**-0.5).bfloat16()
+    y = ops.gemm_skinny(sr, w2.to(DEV)).cpu().float()
+    want = normed @ w2.float().T
+    assert (y - want).abs().max() <= 1.5e-2 * want.abs().max() + 1e-3
+    if F % 8 == 0:
+        wg, wu = (torch.randn(F, N) * N**-0.5).bfloat16(), (torch.randn(F, N) * N**-0.5).bfloat16()
+        act = ops.gemm_skinny(sr, ops.interleave_gate_up(wg, wu).contiguous().to(DEV), silu_mul_epilogue=True).cpu().float()
+        g, u = normed @ wg.float().T, normed @ wu.float().T
+        want = g * torch.sigmoid(g) * u
+        assert (act - want).abs().max() <= 1.5e-2 * want.abs().max() + 1e-3
+    h2 = torch.randn(M, F)
+    h2_d = h2.to(DEV)
+    nw2 = 1 + 0.1 * torch.randn(F)
+    sr2 = ops.gemm_skinny_residual(sr, w2.to(DEV), h2_d, nw2.to(DEV), eps)
+    want_h2 = h2 + normed @ w2.float().T
+    assert torch.allclose(h2_d.cpu(), want_h2, atol=1.5e-2 * float(want_h2.abs().max()))
+    assert sr2.ssq.shape == (M, -(-F // 16))
+
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+def test_gemm_skinny_qkv_on_rows_with_a_norm_to_finish(ops, M):
+    """The q/k/v product on rows that still lack their division by the root mean square: the same
+    queries and cache contents as on the normed rows."""
+    H, KV, hd, P, K = 6, 2, 32, 16, 200
+    torch.manual_seed(M)
+    x = (torch.randn(M, K) * 2).bfloat16()
+    ssq = torch.rand(M, 13) * 50
+    eps = 1e-6
+    w = (torch.randn((H + 2 * KV) * hd, K) * K**-0.5).to(torch.bfloat16)
+    pos = torch.randint(0, 300, (M,), dtype=torch.int32)
+    freqs = plain_rope_frequencies(hd, 10000.0)
+    slots = torch.randperm(4 * P)[:M].to(torch.int32)
+    table = ops.rope_table(pos.to(DEV), freqs.to(DEV))
+    pools = [[torch.zeros((4, KV, P, hd), dtype=torch.bfloat16, device=DEV),
+              torch.zeros((4, KV, hd, P), dtype=torch.bfloat16, device=DEV)] for _ in range(2)]
+    sr = ops.ScaledRows(x.to(DEV), ssq.to(DEV), K, eps)
+    q1 = ops.gemm_skinny_qkv(sr, w.to(DEV), table, slots.to(DEV), *pools[0], H, KV, hd, hd).cpu().float()
+    rstd = torch.rsqrt(ssq.sum(1, keepdim=True) / K + eps)
+    # the reference: the rows scaled in fp32 (the kernel scales the sums, which is the same product)
+    qkv = (x.float() * rstd) @ w.float().T
+    q = plain_rope_interleaved(qkv[:, : H * hd].view(M, H, hd), pos, freqs).reshape(M, -1)
+    assert torch.allclose(q1, q, **tol(torch.bfloat16))
+    k = plain_rope_interleaved(qkv[:, H * hd : (H + KV) * hd].view(M, KV, hd), pos, freqs)
+    v = qkv[:, (H + KV) * hd :].view(M, KV, hd)
+    got_k, got_v = unpack_k(pools[0][0].cpu()).float(), unpack_v(pools[0][1].cpu()).float()
+    for t in range(M):
+        s = int(slots[t])
+        assert torch.allclose(got_k[s // P, :, s % P], k[t], **tol(torch.bfloat16))
+        assert torch.allclose(got_v[s // P, :, s % P], v[t], **tol(torch.bfloat16))
+
+
 # ----------------------------------------------------------------- sampling
 def test_argmax_lowest_index_wins(ops):
     torch.manual_seed(10)
