@@ -52,10 +52,11 @@ class Engine:
     def __init__(self, model: Model, page_size: int = 64, max_tokens: Optional[int] = 8192, max_batch: int = 64,
                  max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0,
                  sync_freq: int = 10, overlap_steps: Optional[bool] = None,
-                 reserve_bytes: Optional[int] = None) -> None:
+                 reserve_bytes: Optional[int] = None, admit_reserve: int = 128) -> None:
         """``max_tokens``: the cache's size in tokens; None: whatever memory the device has free
         now, the weights being in place, beside ``reserve_bytes`` (default: an estimate of what a
-        step of ``max_step_tokens`` tokens and ``max_batch`` rows of logits take, plus 2 GiB)."""
+        step of ``max_step_tokens`` tokens and ``max_batch`` rows of logits take, plus 2 GiB).
+        ``admit_reserve``: tokens of growth that admission keeps room for (see ``Scheduler``)."""
         self.model = model
         cap = getattr(model.args, "max_position", 0) or None
         if max_seq is None:
@@ -67,7 +68,8 @@ class Engine:
         at_most = max_batch * (-(-max_seq // page_size) * page_size) if max_seq else None
         self.runner = ModelRunner(model, page_size=page_size, max_tokens=max_tokens, max_requests=max_batch,
                                   reserve_bytes=reserve_bytes, at_most_tokens=at_most)
-        self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit)
+        self.scheduler = Scheduler(self.runner.cache, max_batch, max_step_tokens, max_seq, on_admit=self.runner.admit,
+                                   admit_reserve=admit_reserve)
         # no request gets longer than the scheduler lets it: block tables need not be wider
         self.runner.table_width = min(self.runner.table_width, -(-self.scheduler.max_seq // page_size))
         self.sampler = Sampler(model.device)

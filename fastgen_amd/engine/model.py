@@ -137,7 +137,7 @@ class Model:
         the cache is written all the same)."""
         if not self.loaded:
             raise RuntimeError("the model has no weights yet")
-        h = self.parts.embed.forward(ctx.tokens)
+        h = self.parts.embed.forward(ctx.tokens, ctx)
         pending = None  # rows still to be added to h, or ScaledRows (added already, the next norm half done)
         blocks, order = self.parts.blocks, self.layout.order
         for i, entry in enumerate(order):

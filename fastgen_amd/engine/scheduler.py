@@ -91,9 +91,19 @@ class PlannedEntry:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_batch: int, max_step_tokens: int,
-                 max_seq: Optional[int] = None, on_admit: Optional[Callable[[Hashable], None]] = None) -> None:
+                 max_seq: Optional[int] = None, on_admit: Optional[Callable[[Hashable], None]] = None,
+                 admit_reserve: int = 128) -> None:
+        """``admit_reserve``: a request is admitted only while the free pages hold, beside its known
+        tokens, this many more of its own and of every running request's tokens still to come (less
+        where a request's cap is nearer).  The reference asks for the prompt and a 128-token buffer
+        at admission (``fastgen/generate.py:535-536, 562``); with it, requests that generate up to
+        128 tokens are never preempted, and longer ones rarely.  0: admit as soon as the known
+        tokens and one more fit."""
         if max_batch < 1 or max_step_tokens < 1:
             raise ValueError("max_batch and max_step_tokens must be at least 1")
+        if admit_reserve < 0:
+            raise ValueError("admit_reserve must not be negative")
+        self.admit_reserve = admit_reserve
         self.cache = cache
         self.max_batch = min(max_batch, cache.n_slots)
         self.max_step_tokens = max_step_tokens
@@ -170,6 +180,22 @@ class Scheduler:
             n = min(n, room)
         return max(0, n)
 
+    def _horizon_pages(self, req: Request) -> int:
+        """Pages of one group that ``req`` holds once it has grown by the admission reserve, or to its cap."""
+        cap = min(len(req.prompt) + req.max_new, self.max_seq)
+        tokens = max(req.n_known() + 1, min(cap, req.n_known() + self.admit_reserve))
+        return -(-tokens // self.cache.page_size)
+
+    def _promised(self) -> List[int]:
+        """Per group: pages that the running requests are still expected to take (see ``admit_reserve``)."""
+        out = [0] * self.cache.n_groups
+        if self.admit_reserve:
+            for r in self.running:
+                want = self._horizon_pages(r)
+                for g in range(self.cache.n_groups):
+                    out[g] += max(0, want - self.cache.n_table_entries(r.rid, g))
+        return out
+
     def plan(self) -> List[PlannedEntry]:
         entries: List[PlannedEntry] = []
         budget = self.max_step_tokens
@@ -220,6 +246,7 @@ class Scheduler:
             entries.append(PlannedEntry(req, req.n_fed, n, n == rem))
             budget -= n
         # C. admission: preempted requests first (they sit at the head), then new ones
+        promised = self._promised() if self.waiting and len(self.running) < self.max_batch and budget > 0 else []
         while self.waiting and len(self.running) < self.max_batch and budget > 0:
             req = self.waiting[0]
             if req.n_pending:  # preempted in this very plan with a sample still on the device: next time
@@ -228,11 +255,18 @@ class Scheduler:
             if any(self.cache.pages_needed_fresh(need, g) > self.cache.free_pages(g)
                    for g in range(self.cache.n_groups)):
                 break
+            # with others running, room for what they and the newcomer are about to grow by as well
+            own = self._horizon_pages(req)
+            if self.running and self.admit_reserve and any(
+                    own + promised[g] > self.cache.free_pages(g) for g in range(self.cache.n_groups)):
+                break
             self.waiting.popleft()
             self._admit(req.rid)
             self.running.append(req)
             n = min(req.remaining(), budget)
             self.cache.reserve(req.rid, n)
+            if self.admit_reserve:  # what it has not taken yet of its horizon is promised to it from here on
+                promised = [p + max(0, own - self.cache.n_table_entries(req.rid, g)) for g, p in enumerate(promised)]
             entries.append(PlannedEntry(req, req.n_fed, n, n == req.remaining()))
             budget -= n
         # D. nothing can move although requests are live: the pages are all

@@ -27,7 +27,9 @@ class Embedding(Part):
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
         self.weight = place(tensors[self._name("weight")], MATRIX, dtype, device)
 
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, ctx: Any = None) -> torch.Tensor:
+        """``ctx`` is the step's context: an embedding that adds something per position (learned or
+        computed absolute positions) finds ``ctx.positions`` there; this one does not look at it."""
         h = torch.empty((tokens.numel(), self.dim), dtype=torch.float32, device=tokens.device)
         return ops.embed(self.weight, tokens, h)
 

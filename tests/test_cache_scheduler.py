@@ -150,9 +150,9 @@ def drive(sched, max_steps=10_000):
     return plans
 
 
-def mk(cache_pages=64, page=16, max_batch=4, budget=24, max_seq=None):
+def mk(cache_pages=64, page=16, max_batch=4, budget=24, max_seq=None, admit_reserve=0):
     c = CacheManager(page, [cache_pages], [None], n_slots=max_batch)
-    return Scheduler(c, max_batch, budget, max_seq)
+    return Scheduler(c, max_batch, budget, max_seq, admit_reserve=admit_reserve)
 
 
 def test_budget_decodes_first_then_prompt_portions():
@@ -505,3 +505,35 @@ def test_a_budget_smaller_than_the_decoding_requests_goes_round():
     assert max(served.values()) - min(served.values()) <= 1, served
     drive(s)
     assert all(len(r.generated) == 12 for r in reqs)
+
+
+def test_admission_keeps_room_for_what_running_requests_will_generate():
+    """The reference asks for the prompt and a 128-token buffer when it admits a request
+    (fastgen/generate.py:535-536): requests that generate no more than the reserve never have to
+    give way.  The same load with and without the reserve: same tokens, preemptions only without."""
+    def load(reserve):
+        s = mk(cache_pages=12, page=16, max_batch=8, budget=256, admit_reserve=reserve)
+        reqs = [Request(i, [i] * 30, max_new=30) for i in range(6)]  # 60 tokens = 4 pages each at the end
+        for r in reqs:
+            s.add(r)
+        return s, reqs
+
+    s0, r0 = load(0)
+    plans0 = drive(s0)
+    assert len(plans0[0]) == 6 and s0.n_preemptions > 0  # all admitted at once: 12 pages; they need 24
+    s1, r1 = load(128)
+    plans1 = drive(s1)
+    assert s1.n_preemptions == 0
+    assert len(plans1[0]) == 3  # three requests of 4 pages each fill the 12 pages
+    for a, b in zip(r0, r1):
+        assert a.generated == b.generated and b.finish_reason == "length"
+    # the reserve is a horizon, not a promise of everything: requests that generate far more than it
+    # are admitted beyond what they will need in the end (and may give way later)
+    s2 = mk(cache_pages=12, page=16, max_batch=8, budget=256, admit_reserve=16)
+    for i in range(6):
+        s2.add(Request(i, [i] * 30, max_new=100, truncate=True))
+    assert len(s2.plan()) == 4  # 46 tokens = 3 pages each
+    # a request alone is admitted as soon as its prompt fits, whatever the reserve
+    s3 = mk(cache_pages=2, page=16, max_batch=2, budget=64, admit_reserve=128)
+    s3.add(Request("a", [1] * 20, max_new=12))
+    assert [e.request.rid for e in s3.plan()] == ["a"]

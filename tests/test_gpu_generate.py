@@ -110,7 +110,7 @@ def test_random_serving_load_matches_the_plain_implementation(seed, tmp_path):
             alone = alone[: alone.index(stop[0]) + 1]
         reqs.append((prompt, SamplingParams(temperature=0.0, max_new_tokens=max_new, stop_ids=stop), alone))
     eng = Engine.from_folder(folder, torch.float32, page_size=16, max_tokens=176, max_batch=5, max_step_tokens=32,
-                             sync_freq=4)
+                             sync_freq=4, admit_reserve=0)
     got = eng.generate([r[0] for r in reqs], [r[1] for r in reqs])
     assert got == [r[2] for r in reqs]
     assert eng.scheduler.n_preemptions > 0
@@ -146,10 +146,14 @@ def test_preemption_gives_the_same_tokens(tiny_b):
     want = roomy.generate(prompts, sp)
     # 12+40+90 prompt tokens and 120 new ones in 15 pages of 16: not all fit at once
     tight = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=16, max_tokens=240, max_batch=3,
-                               max_step_tokens=64)
+                               max_step_tokens=64, admit_reserve=0)
     got = tight.generate(prompts, sp)
     assert tight.scheduler.n_preemptions > 0
     assert got == want
+    # with the admission reserve (the default) the third request waits for room instead: nobody gives way
+    calm = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=16, max_tokens=240, max_batch=3,
+                              max_step_tokens=64)
+    assert calm.generate(prompts, sp) == want and calm.scheduler.n_preemptions == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

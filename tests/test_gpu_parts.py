@@ -163,7 +163,8 @@ class _HybridArch:
             layers.append(LayerSpec(mixer, ffn, norm(f"{p}.n1"), norm(f"{p}.n2"), l.get("arrangement", "pre_norm"),
                                     {name: norm(f"{p}.{name}") for name in l.get("extra_norms", ())}))
         order = tuple(RunEntry(o[0], o[1]) for o in a["order"])
-        return ModelLayout(D, a["vocab"], PartSpec("embedding", "emb", dict(vocab_size=a["vocab"], dim=D)),
+        return ModelLayout(D, a["vocab"], PartSpec(a.get("embedding", "embedding"), "emb",
+                                                   dict(vocab_size=a["vocab"], dim=D, **a.get("embedding_options", {}))),
                            tuple(layers), order, norm("final"),
                            PartSpec("lm_head", "head", dict(vocab_size=a["vocab"], dim=D, tied_to=None)))
 
@@ -176,6 +177,8 @@ def _plain_hybrid(w, a, tokens, mixers, dtype=torch.float32, ffns=None, position
     T = len(tokens)
     w = {k: v.to(dtype) for k, v in w.items()}
     h = w["emb.weight"][torch.tensor(tokens)]
+    if a.get("embedding") == "toy_learned_positions":
+        h = h + w["emb.positions.weight"][:T]
     kv_of = {}
     for idx, (li, src) in enumerate(a["order"]):
         l, p = a["layers"][li], f"blocks.{li}"
@@ -506,3 +509,57 @@ def test_toy_arrangement_with_norms_of_its_own(tmp_path, hybrid_arch):
                 assert_close(run_trace(runner, tr, toks), want, dtype, noise, "sandwich")
     finally:
         unregister_part("arrangement", "toy_sandwich")
+
+
+# ------------------------------------------- positions that enter at the embedding
+def test_toy_embedding_with_learned_positions(tmp_path, hybrid_arch):
+    """A position encoding that is not a rotation inside a mixer: a learned table added to the token
+    embedding, by a toy embedding part registered here.  The step's positions reach it through the
+    context it is handed; the attention layers use the ``none`` position encoding."""
+    from fastgen_amd.engine import Model, ModelRunner
+    from fastgen_amd.kernels import ops
+    from fastgen_amd.parts import Part, TensorSpec, place, register_part, unregister_part
+
+    class LearnedPositions(Part):
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.vocab, self.dim, self.max_pos = spec.options["vocab_size"], spec.options["dim"], spec.options["max_pos"]
+
+        def tensor_specs(self):
+            return [TensorSpec(self._name("weight"), (self.vocab, self.dim)),
+                    TensorSpec(self._name("positions.weight"), (self.max_pos, self.dim))]
+
+        def load(self, tensors, dtype, device):
+            self.weight = place(tensors[self._name("weight")], "matrix", dtype, device)
+            self.positions = place(tensors[self._name("positions.weight")], "matrix", dtype, device)
+
+        def forward(self, tokens, ctx):
+            h = torch.empty((tokens.numel(), self.dim), dtype=torch.float32, device=tokens.device)
+            ops.embed(self.weight, tokens, h)
+            return h.add_(self.positions.index_select(0, ctx.positions.long()).float())  # plain torch: a toy
+
+    register_part("embedding", "toy_learned_positions", LearnedPositions, replace=True)
+    try:
+        args = dict(dim=64, vocab=101, eps=1e-5, theta=1000.0, embedding="toy_learned_positions",
+                    embedding_options=dict(max_pos=80), layers=[
+                        dict(mixer="attention", H=4, KV=2, hd=16, pos="none", F=72),
+                        dict(mixer="attention", H=2, KV=2, hd=32, pos="none", F=40),
+                    ], order=[(0, None), (1, None)])
+        folder, w = _hybrid_case(tmp_path, args)
+        lengths = {"a": 61, "b": 30, "c": 2}
+        g = torch.Generator().manual_seed(9)
+        toks = {r: torch.randint(0, 101, (n,), generator=g).tolist() for r, n in lengths.items()}
+        ident = lambda t, l, a: t  # no rotation
+        want = {r: _plain_hybrid(w, args, t, {}, positions={"none": ident}) for r, t in toks.items()}
+        noise = {r: _plain_hybrid(w, args, t, {}, torch.bfloat16, positions={"none": ident}) for r, t in toks.items()}
+        # without the table the logits are other logits: the positions matter
+        flat = _plain_hybrid({**w, "emb.positions.weight": torch.zeros_like(w["emb.positions.weight"])}, args,
+                             toks["a"], {}, positions={"none": ident})
+        assert (flat - want["a"]).abs().max() > 0.05 * want["a"].abs().max()
+        for dtype in (torch.float32, torch.bfloat16):
+            model = Model.from_folder(folder, dtype, DEV)
+            runner = ModelRunner(model, page_size=16, max_tokens=256, max_requests=3)
+            for tr in (traces.whole(lengths), traces.tail(lengths, 12), traces.mixed(lengths, max_live=3, seed=6)):
+                assert_close(run_trace(runner, tr, toks), want, dtype, noise, "learned positions")
+    finally:
+        unregister_part("embedding", "toy_learned_positions")
