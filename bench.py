@@ -200,13 +200,22 @@ def main() -> int:
     batches = sorted({a.batch} | (set() if a.no_points else {1, 64}))
     max_b = max(batches)
     t0 = time.time()
-    # the cache holds CONTEXT_LEN tokens for every request of the largest batch (68.7 GB at batch 64 of the 8B
-    # shape in bfloat16); with --context beyond it, that many
+    # The cache holds CONTEXT_LEN tokens for every request of the largest batch (68.7 GB at batch 64 of the 8B
+    # shape in bfloat16), or what the GPU has free beside the weights if that is less (the 70B shape); with
+    # --context, as many as the requests reach: the first requests of a batch decode while the prompts of the
+    # later ones are still fed in portions, so they are longer than --context by the number of those steps.
+    from fastgen_amd.engine import Model
+
     ctx_len = a.context or PROMPT_LEN
-    capacity = max(CONTEXT_LEN, -(-(ctx_len + a.warmup + a.steps + 64) // PAGE) * PAGE)
-    engine = Engine.from_config(cfg, seed=2, dtype=dtype, page_size=PAGE,
-                                max_tokens=max_b * capacity, max_batch=max_b,
-                                max_step_tokens=PROMPT_LEN, max_seq=capacity)
+    feed_steps = -(-max_b * ctx_len // max(1, PROMPT_LEN - max_b)) + max_b
+    capacity = max(CONTEXT_LEN, -(-(ctx_len + feed_steps + a.warmup + a.steps + 72) // PAGE) * PAGE)
+    if capacity > cfg["max_position_embeddings"]:
+        print(f"bench.py: --context {ctx_len} and the steps after it pass the model's {cfg['max_position_embeddings']}"
+              " positions", flush=True)
+        return 2
+    model = Model.random(cfg, 2, dtype, "cuda:0")
+    engine = Engine(model, page_size=PAGE, max_tokens=None, max_batch=max_b, max_step_tokens=PROMPT_LEN,
+                    max_seq=capacity)
     torch.cuda.synchronize()
     print(f"[bench] model built in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
     model = engine.model
@@ -237,9 +246,9 @@ def main() -> int:
     for b in batches:
         steps, warm = (a.steps, a.warmup)
         dt = engine.time_decode([prompt(ctx_len) for _ in range(b)], steps=steps, warmup=warm)
-        ctx = ctx_len + warm + steps / 2  # mean cached tokens during the timed steps
+        ctx = engine.last_mean_context  # mean cached tokens of a request during the timed steps
         nbytes = (L * layer_params + D * V) * esize + b * ctx * kv_bytes_per_token
-        results[b] = dict(tok_s=b * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9)
+        results[b] = dict(tok_s=b * steps / dt, ms=dt / steps * 1e3, gbs=nbytes / (dt / steps) / 1e9, ctx=ctx)
         print(f"[bench] decode batch {b}: {results[b]}", file=sys.stderr, flush=True)
 
     r = results[a.batch]
@@ -249,7 +258,7 @@ def main() -> int:
         "ms_per_step": round(r["ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
         "config": {
-            "model": model_name, "global_batch": a.batch, "seq_len": capacity, "mean_context": ctx_len + a.warmup + a.steps / 2,
+            "model": model_name, "global_batch": a.batch, "seq_len": capacity, "mean_context": round(r["ctx"], 1),
             "prompt_len": ctx_len, "cache_tokens": engine.scheduler.pool_tokens, "parallelism": "none", "layers": L, "layers_full": full_layers,
             "hidden": D, "heads": H, "kv_heads": KV, "head_dim": hd, "ffn": F, "vocab": V, "page_size": PAGE,
             "rope_theta": cfg["rope_theta"], "rope_factor": cfg["rope_scaling"]["factor"], "norm_eps": cfg["rms_norm_eps"],

@@ -1,7 +1,7 @@
 """Device tensors behind the cache manager's pages and slots.
 
 Per cache group one K pool ``[n_layers, n_pages, KV, P, hd]`` and one V pool
-``[n_layers, n_pages, KV, hd, P]``: a page of one layer's keys is ``P`` rows of
+``[n_layers, n_pages, KV, hd_v, P]`` (``hd_v`` = ``hd`` unless the group's need says otherwise): a page of one layer's keys is ``P`` rows of
 ``hd`` contiguous elements per head; a page of values is stored transposed so
 that the keys of a page are contiguous for one head dimension.  (The
 reference keeps per layer ``[n_pages*P, KV, hd]`` for both,
@@ -41,7 +41,7 @@ def group_entries(needs: Sequence[Optional[PagedNeed]]) -> List[CacheGroup]:
 def bytes_per_token(groups: Sequence[CacheGroup], dtype: torch.dtype) -> int:
     """Cache bytes one token takes over all layers of all groups."""
     esize = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * len(g.entries) * g.need.n_kv_heads * g.need.head_dim * esize for g in groups)
+    return sum(len(g.entries) * g.need.n_kv_heads * (g.need.head_dim + g.need.value_dim) * esize for g in groups)
 
 
 def tokens_for_free_memory(groups: Sequence[CacheGroup], page_size: int, dtype: torch.dtype,
@@ -80,7 +80,7 @@ class CacheStorage:
             kv, hd = grp.need.n_kv_heads, grp.need.head_dim
             n = len(grp.entries)
             self.k.append(torch.empty((n, n_pages, kv, page_size, hd), dtype=dtype, device=device))
-            self.v.append(torch.empty((n, n_pages, kv, hd, page_size), dtype=dtype, device=device))
+            self.v.append(torch.empty((n, n_pages, kv, grp.need.value_dim, page_size), dtype=dtype, device=device))
             for j, e in enumerate(grp.entries):
                 self._where[e] = (g, j)
         # one row more than there are slots: row ``n_slots`` belongs to nobody.  The stand-in sequences that
@@ -108,7 +108,4 @@ class CacheStorage:
 
     def bytes_per_token(self) -> int:
         """Cache bytes one token takes over all layers (``fastgen/cache.py`` ``bytes_per_token``)."""
-        return sum(
-            2 * len(g.entries) * g.need.n_kv_heads * g.need.head_dim * self.k[i].element_size()
-            for i, g in enumerate(self.groups)
-        )
+        return bytes_per_token(self.groups, self.k[0].dtype) if self.k else 0

@@ -88,6 +88,7 @@ class Engine:
         self._held: List[Request] = []  # ended, with samples still on the device
         self._n_requests = 0
         self.n_steps = 0
+        self.last_mean_context = 0.0  # set by time_decode
 
     # -------------------------------------------------------------- build
     @classmethod
@@ -301,11 +302,16 @@ class Engine:
         run(warmup)
         if len(self.scheduler.running) != len(prompts) or self.scheduler.n_preemptions:
             raise RuntimeError("time_decode: the batch did not stay whole; give the cache more pages")
+        cached = lambda: sum(self.runner.cache.length(r.rid) for r in self.scheduler.running) / len(prompts)
+        before = cached()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         run(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        # tokens a request had in the cache, on average over the requests and the timed steps (the first
+        # requests decoded while the later prompts were fed, so they are longer than their prompts)
+        self.last_mean_context = (before + cached()) / 2
         for r in list(self.scheduler.running):  # the measurement is over: let go of the batch
             self.abort(r.rid)
         self._settle()

@@ -145,7 +145,8 @@ class Fastgen:
         elif gen_args.max_seq < 0:
             if gen_args.gpu_gb > 0:
                 esize = torch.empty((), dtype=gen_args.dtype).element_size()
-                per_token = sum(2 * n.n_kv_heads * n.head_dim * esize for n in model.paged_needs() if n is not None)
+                per_token = sum(n.n_kv_heads * (n.head_dim + n.value_dim) * esize
+                                for n in model.paged_needs() if n is not None)
                 max_tokens = cache_tokens_for_budget(model, gen_args, per_token)
             else:
                 max_tokens = None  # the engine takes what is free

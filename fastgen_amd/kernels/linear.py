@@ -56,11 +56,22 @@ def wide_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[0] <= WIDE_ROWS and _aligned(x, w)
 
 
+_n_cus: Optional[int] = None
+
+
+def _compute_units() -> int:
+    global _n_cus
+    if _n_cus is None:
+        _n_cus = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+    return _n_cus
+
+
 def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
-    """Splits of the k range that give the wide kernel about two workgroups per CU; with many rows
-    a split keeps at least 1,024 of k (the partial sums it writes grow with the rows)."""
+    """Splits of the k range that give the wide kernel (64 output columns a workgroup) about two
+    workgroups per compute unit, at most 8; with many rows a split keeps at least 1,024 of k (the
+    partial sums it writes grow with the rows), else 512.  1: the output is wide enough by itself."""
     blocks = -(-n_out // 64)
-    return max(1, min(8, 512 // blocks, k // (1024 if rows > 48 else 512)))
+    return max(1, min(8, 2 * _compute_units() // blocks, k // (1024 if rows > 48 else 512)))
 
 
 def fold_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -103,9 +114,9 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         return ops.gemm_nt(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
-    if partials_ok and x.shape[0] > 2 and wide_ok(x, w) and w.shape[0] <= 8192:
+    if partials_ok and x.shape[0] > 2 and wide_ok(x, w):
         splits = k_splits_for(w.shape[0], w.shape[1], x.shape[0])
-        if splits > 1:
+        if splits > 3:  # (fewer: the output's own workgroups nearly fill the GPU, partial sums only cost)
             return ops.gemm_skinny(x, w, k_splits=splits, wide=True)
     if skinny_ok(x, w):
         return ops.gemm_skinny(x, w, out_dtype, wide=False)

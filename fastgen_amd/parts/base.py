@@ -49,11 +49,19 @@ def place(t: torch.Tensor, role: str, dtype: torch.dtype, device: torch.device |
 @dataclass(frozen=True)
 class PagedNeed:
     """Per-token storage: keys and values of ``n_kv_heads`` heads of
-    ``head_dim``; with ``window`` only the last ``window`` tokens are read."""
+    ``head_dim``; with ``window`` only the last ``window`` tokens are read.
+    ``v_head_dim``: the width of a value where it differs from a key's (the
+    built-in attention kernels take equal widths only; a mixer with a cache of
+    two widths reads and writes its pages itself)."""
 
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -70,7 +78,7 @@ class LayerStore:
 
     group: Optional[int] = None  # index of its cache group in StepContext.groups
     k_pages: Optional[torch.Tensor] = None  # [n_pages, KV, P, hd]
-    v_pages: Optional[torch.Tensor] = None  # [n_pages, KV, hd, P]
+    v_pages: Optional[torch.Tensor] = None  # [n_pages, KV, hd, P] (hd: the need's value_dim)
     state: Optional[torch.Tensor] = None  # [n_slots, *StateNeed.shape]
     owns: bool = True  # False: the storage belongs to an earlier entry; read only
 

@@ -563,3 +563,25 @@ def test_toy_embedding_with_learned_positions(tmp_path, hybrid_arch):
                 assert_close(run_trace(runner, tr, toks), want, dtype, noise, "learned positions")
     finally:
         unregister_part("embedding", "toy_learned_positions")
+
+
+def test_cache_pools_for_values_of_another_width():
+    """A mixer may ask for values narrower (or wider) than its keys: such a need is a cache group of
+    its own, with a value pool of that width, and counts so in the bytes a token takes.  The built-in
+    attention kernels take equal widths only and say so."""
+    from fastgen_amd.cache.storage import CacheStorage, bytes_per_token, group_entries
+    from fastgen_amd.kernels import KernelArgumentError, ops
+    from fastgen_amd.parts import PagedNeed
+
+    needs = [PagedNeed(2, 32), PagedNeed(2, 32, None, 16), None, PagedNeed(2, 32, None, 16)]
+    groups = group_entries(needs)
+    assert [g.entries for g in groups] == [(0,), (1, 3)]
+    st = CacheStorage(groups, [6, 5], 16, {}, 2, torch.bfloat16, DEV)
+    assert st.k[1].shape == (2, 5, 2, 16, 32) and st.v[1].shape == (2, 5, 2, 16, 16)
+    assert st.bytes_per_token() == bytes_per_token(groups, torch.bfloat16) == (2 * 64 + 2 * 2 * 48) * 2
+    store = st.store_for(3)
+    assert store.group == 1 and store.v_pages.shape == (5, 2, 16, 16)
+    q = torch.zeros(1, 2 * 32, dtype=torch.bfloat16, device=DEV)
+    i = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelArgumentError):
+        ops.paged_attention_general(q, torch.empty_like(q), store.k_pages, store.v_pages, i.view(1, 1), i, i, 2, 1.0)
