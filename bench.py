@@ -169,6 +169,8 @@ def main() -> int:
     ap.add_argument("--shape", choices=sorted(SHAPES), default=None,
                     help="layer sizes: Llama 3.1 8B (the benchmark's configuration; default but for serve), 70B"
                          " (141 GB of weights) or Llama 3.2 3B (the default of serve)")
+    ap.add_argument("--prefill-tokens", type=int, default=PROMPT_LEN,
+                    help="tokens of the timed prefill step (default: the benchmark's 2,048)")
     ap.add_argument("--context", type=int, default=None,
                     help="cached tokens of each request when the timed decode steps begin (default: the prompt's"
                          " 2,048); more are fed untimed, in portions")
@@ -208,7 +210,8 @@ def main() -> int:
 
     ctx_len = a.context or PROMPT_LEN
     feed_steps = -(-max_b * ctx_len // max(1, PROMPT_LEN - max_b)) + max_b
-    capacity = max(CONTEXT_LEN, -(-(ctx_len + feed_steps + a.warmup + a.steps + 72) // PAGE) * PAGE)
+    capacity = max(CONTEXT_LEN, -(-(ctx_len + feed_steps + a.warmup + a.steps + 72) // PAGE) * PAGE,
+                   -(-a.prefill_tokens // PAGE) * PAGE)
     if capacity > cfg["max_position_embeddings"]:
         print(f"bench.py: --context {ctx_len} and the steps after it pass the model's {cfg['max_position_embeddings']}"
               " positions", flush=True)
@@ -232,9 +235,9 @@ def main() -> int:
         return torch.randint(0, V, (n,), generator=g).tolist()
 
     # ------------------------------------------------------------ prefill
-    times = engine.time_prefill(prompt(PROMPT_LEN), repeats=5)
+    times = engine.time_prefill(prompt(a.prefill_tokens), repeats=5)
     pre = sum(times) / len(times)  # the mean of the repeats after one warm-up; the best is reported beside it
-    T = PROMPT_LEN
+    T = a.prefill_tokens
     flops = 2 * T * L * layer_params + L * 4 * H * hd * (T * (T + 1) // 2) + 2 * D * V
     prefill = {"value": round(T / pre, 1), "tokens": T, "ms": round(pre * 1e3, 3),
                "frac": round(flops / pre / PEAK_FLOPS[a.dtype], 4), "repeats": len(times),
