@@ -348,14 +348,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
 // goes through LDS once for all four waves.  blockIdx.y cuts K: split s adds
 // rows k in [s*k_per_split, ...) and stores its partial sums at y + s *
 // part_stride (fp32); the consumer adds the partials in split order.
-// U: k steps of 32 a pass of the loop (8; 4 halves the x slice in LDS and doubles the workgroups a CU
-// holds, which measured no faster at 64 rows).
+// U: k steps of 32 a pass of the loop (8; 4 halves the x slice in LDS, which measured no faster at 64 rows).
+// The x slice has one buffer in LDS (two barriers a pass) and the kernel is held to 170 registers, so that a
+// compute unit holds three workgroups and their loads of W in flight: the gate/up product at 64 rows measured
+// 58.5 us so against 63.5 with two buffers and two workgroups (four workgroups would need 128 registers: spills).
 template <int MB, int U, int EPI, class TY>
-__global__ __launch_bounds__(256, U == 4 ? 4 : 2) void gemm_skinny64_kernel(
+__global__ __launch_bounds__(256, 3) void gemm_skinny64_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
     int ldy, size_t part_stride, int M, int N, int K, int k_per_split) {
-  // [buffer][k chunk][row][8]; row r of chunk c in slot r ^ (c & 15) of its block of 16 (bank conflicts, as above)
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][4 * U * MB * 16 * 8];
+  // [k chunk][row][8]; row r of chunk c in slot r ^ (c & 15) of its block of 16 (bank conflicts, as above)
+  __shared__ __attribute__((aligned(16))) bf16_t xs[4 * U * MB * 16 * 8];
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 64 + wave * 16;
@@ -386,15 +388,15 @@ __global__ __launch_bounds__(256, U == 4 ? 4 : 2) void gemm_skinny64_kernel(
     }
   };
   if (k_begin < k_end) fetch(k_begin);
-  int buf = 0;
-  for (int kk = k_begin; kk < k_end; kk += 32 * U, buf ^= 1) {
-    bf16_t* my = xs[buf];
+  for (int kk = k_begin; kk < k_end; kk += 32 * U) {
+    bf16_t* my = xs;
+    __syncthreads();  // the slice of the pass before is no longer read
 #pragma unroll
     for (int j = 0; j < XL; ++j) *(bf16x8*)(my + (c_chunk * (MB * 16) + ((c_row + RP * j) ^ (c_chunk & 15))) * 8) = xv[j];
     bf16x8 a[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) a[u] = a_next[u];
-    __syncthreads();  // this buffer is complete; the other one may still be read by slower waves
+    __syncthreads();  // the slice is complete
     if (kk + 32 * U < k_end) fetch(kk + 32 * U);
 #pragma unroll
     for (int u = 0; u < U; ++u)
