@@ -12,6 +12,7 @@ meanings of options where the reference has them.
 from __future__ import annotations
 
 import logging
+import os
 import queue
 from dataclasses import dataclass, field
 from pathlib import Path
@@ -106,6 +107,17 @@ class HfLoader:
 class Fastgen:
     def __init__(self, engine: Engine, gen_args: GenArgs, stop_tokens: Sequence[int] = ()) -> None:
         self.engine, self.gen_args, self.stop_tokens = engine, gen_args, tuple(stop_tokens)
+        # A trace on request (``fastgen/generate.py:187-196, 364-403``): ``request_profile()``, or the signal
+        # SIGUSR2 where ``build`` could install its handler, starts ``torch.profiler`` at the top of the next
+        # iteration of the generation loop; after FG_PROFILE_ITERS iterations (default 8) a chrome trace is
+        # written to FG_PROFILE_DIR (default /tmp) as fastgen_<pid>_<HHMMSS.f>.json.gz.
+        self.profile_state = "inactive"  # inactive / requested / active
+        self.profile_iter = 0
+        self.profile_iters = int(os.environ.get("FG_PROFILE_ITERS", "8"))
+        self.profile_dir = os.environ.get("FG_PROFILE_DIR", "/tmp")
+        self.last_profile: Optional[str] = None  # the trace written last
+        self._profile_ctx: Any = None
+        self._profile_obj: Any = None
 
     @classmethod
     def build(cls, loader: "HfLoader | str | Path", gen_args: GenArgs = GenArgs(), tp_mesh: Any = None,
@@ -160,7 +172,61 @@ class Fastgen:
         logger.info("cache of %d tokens in pages of %d, at most %d requests",
                     engine.scheduler.pool_tokens, gen_args.cache_block, engine.scheduler.max_batch)
         engine.runner.max_graphs = max(0, gen_args.num_cuda_graphs)
-        return cls(engine, gen_args, stop_tokens)
+        fg = cls(engine, gen_args, stop_tokens)
+        fg._install_profile_signal()
+        return fg
+
+    # ---------------------------------------------------------- profiling
+    def _install_profile_signal(self, signum: Optional[int] = None) -> None:
+        """SIGUSR2 requests a trace, if nobody else handles that signal (generate.py:165-172) and this
+        is the main thread (only there can a handler be set)."""
+        import signal
+        import threading
+
+        signum = signal.SIGUSR2 if signum is None else signum
+        if threading.current_thread() is not threading.main_thread():
+            return
+        if signal.getsignal(signum) is not signal.SIG_DFL:
+            logger.warning("a handler for signal %s is set; the profile handler was not installed", signum)
+            return
+        signal.signal(signum, lambda _signum, _frame: self.request_profile())
+
+    def request_profile(self) -> None:
+        """Ask for a trace of the next ``FG_PROFILE_ITERS`` iterations of the generation loop."""
+        if self.profile_state == "inactive":
+            logger.info("profile trace requested")
+            self.profile_state = "requested"
+
+    def _profile_step(self) -> None:
+        if self.profile_state == "active":
+            self.profile_iter += 1
+            if self.profile_iter >= self.profile_iters:
+                self._profile_done()
+            return
+        from torch.profiler import ProfilerActivity, profile
+
+        self.profile_iter = 0
+        self._profile_ctx = profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA], with_stack=True)
+        self._profile_obj = self._profile_ctx.__enter__()
+        self.profile_state = "active"
+
+    def _profile_done(self, dump: bool = True) -> None:
+        if self.profile_state != "active":
+            return
+        self.profile_state = "inactive"
+        try:
+            self._profile_ctx.__exit__(None, None, None)
+            if dump:
+                from datetime import datetime
+
+                path = f"{self.profile_dir}/fastgen_{os.getpid()}_{datetime.now().strftime('%H%M%S.%f')}.json.gz"
+                self._profile_obj.export_chrome_trace(path)
+                self.last_profile = path
+                logger.info("profile chrome trace exported to %s", path)
+        except Exception as e:  # a trace that cannot be written must not end the generation
+            logger.warning("error while exporting the profile trace: %r", e)
+        finally:
+            self._profile_ctx = self._profile_obj = None
 
     def _params(self, pkt: Packet) -> SamplingParams:
         ga = self.gen_args
@@ -181,6 +247,8 @@ class Fastgen:
         pending = {}
         refused: List[Packet] = []
         while True:
+            if self.profile_state != "inactive":
+                self._profile_step()
             while not eoq:
                 try:
                     pkt = q.get(block=not self.engine.has_work())
@@ -203,6 +271,7 @@ class Fastgen:
                 yield refused.pop(0)
             if not self.engine.has_work():
                 if eoq:
+                    self._profile_done()  # a trace that was still running is written with what it has
                     return
                 continue
             for req in self.engine.step():

@@ -3,6 +3,7 @@ implementation, sampling with seeds, preemption, the reference-style
 interface and the command line."""
 
 import json
+import os
 import queue
 import subprocess
 import sys
@@ -560,3 +561,40 @@ def test_command_line_with_random_weights_and_pages(tiny_b, tmp_path):
     assert len(d) == 28 and d[:12] == a
     proc = subprocess.run(base[:2] + ["--prompt-ids", "1"], capture_output=True, text=True, timeout=60)
     assert proc.returncode == 2 and "--random-weights" in proc.stderr
+
+
+def test_profile_trace_on_request(tiny_b, tmp_path, monkeypatch):
+    """``request_profile()`` (the reference's hook, also bound to SIGUSR2): the next FG_PROFILE_ITERS
+    iterations of the generation loop are traced and a chrome trace is written to FG_PROFILE_DIR; the
+    generation itself is not disturbed."""
+    import gzip
+    import signal
+
+    from fastgen_amd.generate import Fastgen, GenArgs, Packet
+
+    monkeypatch.setenv("FG_PROFILE_ITERS", "3")
+    monkeypatch.setenv("FG_PROFILE_DIR", str(tmp_path))
+    old = signal.getsignal(signal.SIGUSR2)
+    try:
+        fg = Fastgen.build(tiny_b["folder"], GenArgs(use_sampling=False, max_batch=2, max_seq=512, max_gen=12,
+                                                    cache_block=32, dtype=torch.bfloat16, sync_freq=2), stop_tokens=())
+        assert fg.profile_iters == 3 and fg.profile_state == "inactive"
+        if old is signal.SIG_DFL:  # nobody else handled it: the signal asks for a trace
+            os.kill(os.getpid(), signal.SIGUSR2)
+        else:
+            fg.request_profile()
+        assert fg.profile_state == "requested"
+        q = queue.Queue()
+        for i in (1, 2):
+            q.put(Packet(thread_id=i, tokens=tiny_b["prompts"][i]))
+        q.put(None)
+        out = {p.thread_id: p.tokens for p in fg.generate(q)}
+        assert len(out[1]) == len(out[2]) == 12
+        assert fg.profile_state == "inactive" and fg.last_profile is not None
+        traces_ = list(tmp_path.glob("fastgen_*.json.gz"))
+        assert len(traces_) == 1 and str(traces_[0]) == fg.last_profile
+        with gzip.open(traces_[0], "rt") as f:
+            text = f.read()
+        assert "traceEvents" in text and ("gemm_skinny" in text or "attn_" in text)  # the engine's kernels are in it
+    finally:
+        signal.signal(signal.SIGUSR2, old)
