@@ -69,6 +69,16 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 #define LOG2E 1.4426950408889634f
 
+// Maximum over the four lanes that hold one query row (lane % 16 in each group of 16), in every one
+// of them.  gfx950 swaps rows of 16 and halves of 32 lanes between two registers in the vector unit
+// (no trip through the LDS crossbar, whose latency a wave with one or two row blocks cannot hide).
+__device__ __forceinline__ float max_over_groups(float v) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));  // rows 0|1 and 2|3
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));  // halves
+}
+
 // key (within a tile) of S^T row `row` (0..15) of key block kb (0..3)
 __device__ __forceinline__ int key_of(int kb, int row) { return 16 * kb + row; }
 
@@ -160,8 +170,7 @@ __device__ __forceinline__ void attend_tile(int k0, const ItemRows (&me)[RB], co
         s[rb][kb][i] = v;
         mx = fmaxf(mx, v);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, FG_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, FG_WAVE));
+    mx = max_over_groups(mx);
     const float m_new = fmaxf(m[rb], mx * scale_log2);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
     const float alpha = __builtin_amdgcn_exp2f(m[rb] - m_use);  // m = -inf: 0
