@@ -1,4 +1,4 @@
-// y = x W^T for few rows of x (decode: M <= 64), bf16 operands, fp32
+// y = x W^T for few rows of x (decode: M <= 128), bf16 operands, fp32
 // accumulation on the matrix cores.  The work is streaming W once from HBM,
 // so the kernel is built around keeping many 16-byte loads of W in flight:
 //
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
   }
 }
 
-// More rows of x (17..64): a workgroup owns 64 rows of W, one 16-row block a
+// More rows of x (17..128): a workgroup owns 64 rows of W, one 16-row block a
 // wave over the whole k range of the workgroup, so nothing is reduced across
 // waves; the workgroup's slice of x for the next 8 k steps (MB*16 rows x 256)
 // goes through LDS once for all four waves.  blockIdx.y cuts K: split s adds
@@ -352,8 +352,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
 // The x slice has one buffer in LDS (two barriers a pass) and the kernel is held to 170 registers, so that a
 // compute unit holds three workgroups and their loads of W in flight: the gate/up product at 64 rows measured
 // 58.5 us so against 63.5 with two buffers and two workgroups (four workgroups would need 128 registers: spills).
+// Above 64 rows (five to eight blocks of x: two workgroups a compute unit) every wave reads eight blocks of x from
+// LDS for each 16 rows of W, which bounds it: worth it where the k range is cut (down and o projections at 128
+// rows of the 8B shape 46 / 18 us against the library's 76 / 24), not for wide outputs (gate/up 75 against 55).
 template <int MB, int U, int EPI, class TY>
-__global__ __launch_bounds__(256, 3) void gemm_skinny64_kernel(
+__global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
     int ldy, size_t part_stride, int M, int N, int K, int k_per_split) {
   // [k chunk][row][8]; row r of chunk c in slot r ^ (c & 15) of its block of 16 (bank conflicts, as above)
@@ -510,14 +513,14 @@ extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int l
   return fg_launch_status();
 }
 
-// x [M, K] bf16 with 16 < M <= 64 (fewer rows work too).  k_splits > 1: y is fp32 [k_splits, M, N]
+// x [M, K] bf16 with 16 < M <= 128 (fewer rows work too).  k_splits > 1: y is fp32 [k_splits, M, N]
 // (part_stride elements apart), partial sums over K to be added by the consumer in split order;
 // only with epilogue 0.
 extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, void* y, int ldy,
                                 long long part_stride, int k_splits, int M, int N, int K, int out_dtype,
                                 int epilogue, hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
-  if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535)
+  if (M > 128 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535)
     return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
@@ -526,7 +529,7 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   const dim3 grid((N + 63) / 64, k_splits);
   const int mb = (M + 15) / 16;
 #define GO64(MB, EPI, TY)                                                                                    \
-  gemm_skinny64_kernel<MB, 8, EPI, TY><<<grid, 256, 0, stream>>>(                             \
+  gemm_skinny64_kernel<MB, 8, EPI, TY><<<grid, 256, 0, stream>>>(                                             \
       (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split)
 #define PICK(MB)                                                                   \
   do {                                                                             \
@@ -538,7 +541,11 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   if (mb == 1) PICK(1);
   else if (mb == 2) PICK(2);
   else if (mb == 3) PICK(3);
-  else PICK(4);
+  else if (mb == 4) PICK(4);
+  else if (mb == 5) PICK(5);
+  else if (mb == 6) PICK(6);
+  else if (mb == 7) PICK(7);
+  else PICK(8);
 #undef PICK
 #undef GO64
   return fg_launch_status();

@@ -3,9 +3,11 @@
 float32: the engine's own fused-multiply-add kernel (``gemm.hip``), a true
 32-bit product whose rows do not depend on one another.  bfloat16: up to 16
 rows (decode) the engine's weight-streaming MFMA kernel (``gemm_skinny.hip``);
-more rows the vendor library's matrix product through ``torch`` (the reference
-uses cuBLAS through ``F.linear`` for all of them, ``fastgen/forward.py:433-513``),
-with fp32 accumulation; logits are asked for in fp32 directly.
+up to 64 rows (128 where the k range is cut) its wider sibling where that beats
+the library; otherwise the vendor library's matrix product through ``torch`` (the
+reference uses cuBLAS through ``F.linear`` for all of them,
+``fastgen/forward.py:433-513``), with fp32 accumulation; logits are asked for in
+fp32 directly.
 """
 
 from __future__ import annotations
@@ -38,6 +40,8 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
 # up to this many rows the weight-streaming kernels are used (more: the library's product)
 SKINNY_ROWS = 16  # one 16-row block of x, 16 output columns a workgroup
 WIDE_ROWS = 64    # up to four blocks of x, 64 output columns a workgroup
+FUSED_GATE_UP_ROWS = 80
+TALL_ROWS = 128   # with k splits (few output columns, long k) the same kernel with up to eight blocks of x
 
 
 def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -51,9 +55,16 @@ def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return x.shape[0] <= SKINNY_ROWS and _aligned(x, w)
 
 
-def wide_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Up to 64 rows: the engine's kernel where it beats the library (fused epilogue, or k splits)."""
-    return x.shape[0] <= WIDE_ROWS and _aligned(x, w)
+def fused_gate_up_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """The gate/up product with ``silu(gate) * up`` in its epilogue, where that beats the library's product plus
+    an activation kernel: up to 80 rows (8B shape at 80 rows: 63 us against 64 + 8; at 96 rows 66 against 54 + 8)."""
+    return x.shape[0] <= FUSED_GATE_UP_ROWS and _aligned(x, w)
+
+
+def tall_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Up to 128 rows, for a product whose k range is cut (the o and down projections: the library runs them as
+    32 tiles of 128 columns without a cut, 76 / 24 us at 128 rows of the 8B shape against 46 / 18)."""
+    return x.shape[0] <= TALL_ROWS and _aligned(x, w)
 
 
 _n_cus: Optional[int] = None
@@ -114,7 +125,7 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         return ops.gemm_nt(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
-    if partials_ok and x.shape[0] > 2 and wide_ok(x, w):
+    if partials_ok and x.shape[0] > 2 and tall_ok(x, w):
         splits = k_splits_for(w.shape[0], w.shape[1], x.shape[0])
         if splits > 3:  # (fewer: the output's own workgroups nearly fill the GPU, partial sums only cost)
             return ops.gemm_skinny(x, w, k_splits=splits, wide=True)

@@ -456,7 +456,7 @@ def gemm_nt(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None
     return out
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 128
 
 
 @dataclass
@@ -534,14 +534,14 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, h: torch.Tensor, norm
 
 def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 silu_mul_epilogue: bool = False, k_splits: int = 1, wide: Optional[bool] = None) -> torch.Tensor:
-    """``x @ w.T`` for at most 64 rows of bf16 ``x`` on the matrix cores, built to
+    """``x @ w.T`` for at most 128 rows of bf16 ``x`` on the matrix cores, built to
     stream ``w [N, K]`` once.  ``x`` may be :class:`ScaledRows` (at most 16 rows, bfloat16 out): the
     result rows are scaled.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
     ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
     ``[M, N/2]``.  With ``k_splits > 1`` the k range is cut over workgroups and the
     result is fp32 ``[k_splits, M, N]`` partial sums (for few output columns,
     where one workgroup per 64 columns would leave most of the GPU idle).
-    ``wide`` picks the kernel for 17..64 rows (64 columns a workgroup, x shared
+    ``wide`` picks the kernel for 17..128 rows (64 columns a workgroup, x shared
     through LDS); default: by the number of rows."""
     scaled = x if isinstance(x, ScaledRows) else None
     if scaled is not None:
@@ -558,6 +558,7 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     if silu_mul_epilogue:
         _need(N % 16 == 0 and out_dtype == torch.bfloat16, "the gate/up epilogue needs N % 16 == 0 and bf16 output")
     wide = (M > 16 or k_splits > 1) if wide is None else wide
+    _need(M <= 64 or wide, "more than 64 rows take the wide kernel")
     _need(k_splits >= 1 and (k_splits == 1 or (wide and not silu_mul_epilogue)), "k_splits needs the wide kernel")
     if k_splits > 1:
         out_dtype = torch.float32

@@ -11,7 +11,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear, skinny_ok, wide_ok
+from ..kernels.linear import fused_gate_up_ok, linear, skinny_ok
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
@@ -51,7 +51,7 @@ class SwiGLU(FeedForward):
         rows = x.rows if isinstance(x, ops.ScaledRows) else x
         if rows is not x and not skinny_ok(rows, self.w_gate_up):
             x = rows = x.materialize()
-        if wide_ok(rows, self.w_gate_up):
+        if fused_gate_up_ok(rows, self.w_gate_up):
             act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True)
         else:
             act = ops.silu_mul(linear(x, self.w_gate_up))

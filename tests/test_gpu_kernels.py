@@ -345,7 +345,7 @@ def test_gemm_skinny(ops, M, N, K, odtype):
     assert err < (1e-5 if odtype == torch.float32 else 6e-3), float(err)
 
 
-@pytest.mark.parametrize("M", [1, 8, 17, 40, 64])
+@pytest.mark.parametrize("M", [1, 8, 17, 40, 64, 65, 83, 128])
 @pytest.mark.parametrize("N,K,S", [(515, 240, 1), (4096, 4096, 4), (4096, 14336, 8), (100, 264, 3), (6144, 64, 1)])
 def test_gemm_skinny_wide_and_k_splits(ops, M, N, K, S):
     torch.manual_seed(17)
@@ -392,7 +392,9 @@ def test_gemm_skinny_takes_views_and_refuses_the_rest(ops):
     got = ops.gemm_skinny(x, w).cpu().float()
     assert torch.allclose(got, x.cpu().float() @ w.cpu().float().T, atol=0.3, rtol=2e-2)
     with pytest.raises(KernelArgumentError, match="rows"):
-        ops.gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+        ops.gemm_skinny(torch.zeros(129, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    with pytest.raises(KernelArgumentError, match="wide"):
+        ops.gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous(), wide=False)
     with pytest.raises(KernelArgumentError, match="multiple of 8"):
         ops.gemm_skinny(torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV),
                         torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV))
