@@ -237,7 +237,10 @@ __device__ __forceinline__ void item_tiles(const Item& it, int window, int& t_lo
 }
 
 // One workgroup.  Tiles per chunk: the smallest multiple of min_tiles (at least min_tiles) with which
-// all chunks fit into max_chunks (> n_items) and no item has more than COMBINE_MAX_SPLITS.
+// all chunks fit into max_chunks (> n_items) whatever the items' lengths are (total / (max_chunks -
+// n_items), rounded up) and no item has more than COMBINE_MAX_SPLITS; then, with the number of chunks
+// that this gives the longest item, as even as they can be (33 tiles in chunks of 12, 12, 9, not 16,
+// 16, 1: sequences of one length are the common case), if the chunks of all items still fit.
 __global__ __launch_bounds__(256) void attn_plan_kernel(const int* __restrict__ items, int n_items, int window,
                                                         int max_chunks, int min_tiles, int* __restrict__ plan) {
   __shared__ int red_s[256], red_m[256];
@@ -267,6 +270,24 @@ __global__ __launch_bounds__(256) void attn_plan_kernel(const int* __restrict__ 
   const int room = max_chunks - n_items;
   int ts = max((tot + room - 1) / room, (mx + COMBINE_MAX_SPLITS - 1) / COMBINE_MAX_SPLITS);
   ts = max(1, (ts + min_tiles - 1) / min_tiles) * min_tiles;
+  const int longest_chunks = max(1, (mx + ts - 1) / ts);  // chunks of the longest item
+  const int even = max(1, ((mx + longest_chunks - 1) / longest_chunks + min_tiles - 1) / min_tiles) * min_tiles;
+  if (even < ts) {  // uniform
+    int cnt = 0;
+    for (int i = tid; i < n_items; i += 256) {
+      int lo, hi;
+      item_tiles(load_item(items, i), window, lo, hi);
+      cnt += (hi - lo + even) / even;
+    }
+    red_s[tid] = cnt;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if (tid < w) red_s[tid] += red_s[tid + w];
+      __syncthreads();
+    }
+    if (red_s[0] <= max_chunks) ts = even;
+    __syncthreads();
+  }
   int* chunks = plan + PLAN_HEAD;
   if (tid == 0) carry = 0;
   __syncthreads();

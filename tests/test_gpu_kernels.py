@@ -708,6 +708,7 @@ def test_paged_attention_mfma_many_decoding_sequences(ops, n_items, cut):
 
 @pytest.mark.parametrize("n_items,window,max_chunks,min_tiles", [
     (1, 0, 2, 4), (7, 0, 128, 4), (7, 100, 14, 1), (300, 0, 600, 4), (300, 777, 1024, 1), (513, 0, 4096, 2),
+    (8, 0, 40, 4), (12, 0, 44, 4), (40, 0, 81, 2),
 ])
 def test_attention_plan_cuts_every_item_into_equal_chunks(ops, n_items, window, max_chunks, min_tiles):
     """The plan that the split kernel works from: every item's tiles are covered once, in order, by
@@ -738,9 +739,14 @@ def test_attention_plan_cuts_every_item_into_equal_chunks(ops, n_items, window, 
             assert rec[4] == t_lo + c * ts and rec[5] == min(t_hi + 1, t_lo + (c + 1) * ts)
         nxt += count
     assert nxt == used
-    # coarser is never needed: with chunks one step smaller the list would overflow, or it is the least allowed
-    if ts > min_tiles:
-        smaller = ts - min_tiles
-        tiles = [(pos0[i] + n_tok[i] - 1) // 64 - ((max(0, pos0[i] - window + 1) if window else 0) // 64) + 1
-                 for i in range(n_items)]
-        assert sum(tiles) / smaller + n_items > max_chunks or max(tiles) > 256 * smaller
+    # the size that fits whatever the lengths are; with the longest item's number of chunks at that size, as even
+    # as they can be, if all items' chunks still fit
+    tiles = np.array([(pos0[i] + n_tok[i] - 1) // 64 - ((max(0, pos0[i] - window + 1) if window else 0) // 64) + 1
+                      for i in range(n_items)])
+    up = lambda v: max(1, -(-v // min_tiles)) * min_tiles
+    longest = int(tiles.max())
+    want = up(max(-(-int(tiles.sum()) // (max_chunks - n_items)), -(-longest // 256)))
+    even = up(-(-longest // -(-longest // want)))
+    if even < want and int((-(-tiles // even)).sum()) <= max_chunks:
+        want = even
+    assert ts == want
