@@ -52,12 +52,12 @@ def test_family_shape_under_every_cut(family, dtype):
             assert_close(got, family["plain32"], dtype, family["noise16"], name)
 
 
-@pytest.mark.parametrize("n_live", [24, 61, 100])
+@pytest.mark.parametrize("n_live", [24, 61, 75, 100])
 def test_family_shape_many_requests_decode_together(family, n_live):
     """The benchmark's decode path at its layer sizes: dozens of live requests of different lengths,
     prompts fed in portions, then 40 decode steps of all together, eagerly and from captured steps
-    (61 requests in a step recorded for 64, 100 in one for 128): the wide products with k splits at
-    17..64 rows and, for o and down, at 65..128, the library's q/k/v product with the rotation kernel,
+    (61 requests in a step recorded for 64, 75 in one for 80, 100 in one for 128): the wide products with k splits at
+    17..64 rows and, for o and down, at 65..128 (gate/up with its activation up to 80), the library's q/k/v product with the rotation kernel,
     split attention with dozens of items and both combine kernels.  Every position against the plain implementation, which for this many tokens
     runs its torch operations on the GPU; that run is pinned to the CPU run on one request."""
     import numpy as np

@@ -370,7 +370,7 @@ def test_gemm_skinny_wide_and_k_splits(ops, M, N, K, S):
         assert (got.cpu().double() - want).abs().max() / want.abs().max() < 6e-3
 
 
-@pytest.mark.parametrize("M", [17, 64])
+@pytest.mark.parametrize("M", [17, 64, 65, 80, 128])
 def test_gemm_skinny_wide_gate_up(ops, M):
     torch.manual_seed(18)
     F, K = 1000, 328
