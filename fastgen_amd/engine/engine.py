@@ -11,7 +11,7 @@ import os
 import time
 from dataclasses import dataclass
 from pathlib import Path
-from typing import Any, Dict, Hashable, Iterable, List, Mapping, Optional, Sequence
+from typing import Any, Dict, Hashable, List, Mapping, Optional, Sequence
 
 import torch
 

@@ -14,7 +14,6 @@ import sys
 from pathlib import Path
 from typing import IO, Optional
 
-import numpy as np
 import torch
 
 from ..config import read_config_json

@@ -11,9 +11,8 @@ is one, because a decoded token is a portion of length one.
 from __future__ import annotations
 
 import os
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, Optional, Sequence, Tuple
 
-import numpy as np
 import torch
 
 from ..cache.manager import CacheManager

@@ -39,7 +39,6 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
 
 # up to this many rows the weight-streaming kernels are used (more: the library's product)
 SKINNY_ROWS = 16  # one 16-row block of x, 16 output columns a workgroup
-WIDE_ROWS = 64    # up to four blocks of x, 64 output columns a workgroup
 FUSED_GATE_UP_ROWS = 80
 TALL_ROWS = 128   # with k splits (few output columns, long k) the same kernel with up to eight blocks of x
 

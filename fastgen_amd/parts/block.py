@@ -3,7 +3,7 @@ the residual stream."""
 
 from __future__ import annotations
 
-from typing import Any, Optional, Tuple
+from typing import Any, Optional
 
 import torch
 
