@@ -358,9 +358,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
 template <int MB, int U, int EPI, class TY>
 __global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
     const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict__ w, int ldw, TY* __restrict__ y,
-    int ldy, size_t part_stride, int M, int N, int K, int k_per_split) {
+    int ldy, size_t part_stride, int M, int N, int K, int k_per_split, RowScale sc) {
   // [k chunk][row][8]; row r of chunk c in slot r ^ (c & 15) of its block of 16 (bank conflicts, as above)
   __shared__ __attribute__((aligned(16))) bf16_t xs[4 * U * MB * 16 * 8];
+  __shared__ float rscale[16];  // with sc (one block of x only): the rows' factors of a norm folded into this product
+  const float sc_part = MB == 1 ? row_scale_begin<256>(sc, M) : 0.f;
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 64 + wave * 16;
@@ -411,6 +413,11 @@ __global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
   }
   // acc[mb][i] = C[n = n0 + 4g + i][m = 16 mb + r16]
   TY* yp = y + (size_t)blockIdx.y * part_stride;
+  if (MB == 1 && sc.ssq) {  // uniform
+    row_scale_end<256>(sc, sc_part, rscale);
+    __syncthreads();
+    acc[0] *= rscale[r16];
+  }
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int m = 16 * mb + r16;
@@ -516,10 +523,15 @@ extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int l
 // x [M, K] bf16 with 16 < M <= 128 (fewer rows work too).  k_splits > 1: y is fp32 [k_splits, M, N]
 // (part_stride elements apart), partial sums over K to be added by the consumer in split order;
 // only with epilogue 0.
+// ssq [M, n_parts] (null: x is taken as it is; else M <= 16 and one split): the rows' sums of squares for a norm
+// folded into this product, dim = the width that they run over.
 extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, void* y, int ldy,
                                 long long part_stride, int k_splits, int M, int N, int K, int out_dtype,
-                                int epilogue, hipStream_t stream) {
+                                int epilogue, const float* ssq, int n_parts, int dim, float eps,
+                                hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
+  if (ssq && (M > 16 || k_splits != 1 || n_parts < 1 || dim < 1 || !(eps >= 0.f))) return FG_ERR_ARG;
+  const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
   if (M > 128 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535)
     return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
@@ -530,7 +542,7 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   const int mb = (M + 15) / 16;
 #define GO64(MB, EPI, TY)                                                                                    \
   gemm_skinny64_kernel<MB, 8, EPI, TY><<<grid, 256, 0, stream>>>(                                             \
-      (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split)
+      (const bf16_t*)x, ldx, (const bf16_t*)w, ldw, (TY*)y, ldy, (size_t)part_stride, M, N, K, k_per_split, sc)
 #define PICK(MB)                                                                   \
   do {                                                                             \
     if (epilogue == EPI_SILU_MUL) GO64(MB, EPI_SILU_MUL, bf16_t);                  \

@@ -542,7 +542,7 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     result is fp32 ``[k_splits, M, N]`` partial sums (for few output columns,
     where one workgroup per 64 columns would leave most of the GPU idle).
     ``wide`` picks the kernel for 17..128 rows (64 columns a workgroup, x shared
-    through LDS); default: by the number of rows."""
+    through LDS; it takes fewer rows and ``ScaledRows`` too); default: by the number of rows."""
     scaled = x if isinstance(x, ScaledRows) else None
     if scaled is not None:
         x = scaled.rows
@@ -565,8 +565,13 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     cols = N // 2 if silu_mul_epilogue else N
     y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
     lib = _lib.load("gemm_skinny")
-    if scaled is not None:
-        _need(M <= 16 and not wide and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
+    if scaled is not None and wide:
+        _need(M <= 16 and k_splits == 1 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
+        st = lib.fg_gemm_skinny64(
+            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), 1, M, N,
+            K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(scaled, M), _stream(x))
+    elif scaled is not None:
+        _need(M <= 16 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
         st = lib.fg_gemm_skinny_fused(
             _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, 1 if silu_mul_epilogue else 0,
             *_row_scale_args(scaled, M), ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0,
@@ -574,7 +579,7 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     elif wide:
         st = lib.fg_gemm_skinny64(
             _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
-            K, _code(y), 1 if silu_mul_epilogue else 0, _stream(x))
+            K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(None, M), _stream(x))
     else:
         st = lib.fg_gemm_skinny(
             _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, _code(y),

@@ -52,7 +52,10 @@ class SwiGLU(FeedForward):
         if rows is not x and not skinny_ok(rows, self.w_gate_up):
             x = rows = x.materialize()
         if fused_gate_up_ok(rows, self.w_gate_up):
-            act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True)
+            # from 11 rows on the wide kernel (64 columns a workgroup, x through LDS) is the faster one for this
+            # product's many columns (8B shape: a decode step of 12 / 14 / 16 sequences 4.60 / 4.71 / 4.80 ms
+            # against 4.67 / 4.84 / 5.00; equal at 10, slower at 9)
+            act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True, wide=rows.shape[0] > 10)
         else:
             act = ops.silu_mul(linear(x, self.w_gate_up))
         return linear(act, self.w_down, partials_ok=True, residual=then)

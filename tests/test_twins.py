@@ -300,8 +300,12 @@ def test_gemm_skinny_twins(ops, M, N, K):
     if M <= 16:
         folded_c = twins.gemm_skinny_residual(x, w, h.clone(), norm_w, 1e-5)
         folded_g = kernel_ops.ScaledRows(folded_c.rows.cuda(), folded_c.ssq.cuda(), folded_c.dim, folded_c.eps)
-        w2 = (torch.randn(40, N) / 4).to(bf)
+        w2 = (torch.randn(48, N) / 4).to(bf)
         _close(ops.gemm_skinny(folded_g, w2.cuda()), twins.gemm_skinny(folded_c, w2), bf)
+        for wide in (False, True):  # the norm's factor in either kernel, with and without the gate/up epilogue
+            _close(ops.gemm_skinny(folded_g, w2.cuda(), wide=wide), twins.gemm_skinny(folded_c, w2, wide=wide), bf)
+            _close(ops.gemm_skinny(folded_g, w2.cuda(), None, True, 1, wide),
+                   twins.gemm_skinny(folded_c, w2, None, True, 1, wide), bf)
 
 
 @gpu
