@@ -40,6 +40,7 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
 # up to this many rows the weight-streaming kernels are used (more: the library's product)
 SKINNY_ROWS = 16  # one 16-row block of x, 16 output columns a workgroup
 FUSED_GATE_UP_ROWS = 80
+LOGITS_SKINNY_ROWS = 8
 TALL_ROWS = 128   # with k splits (few output columns, long k) the same kernel with up to eight blocks of x
 
 
@@ -128,7 +129,9 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         splits = k_splits_for(w.shape[0], w.shape[1], x.shape[0])
         if splits > 3:  # (fewer: the output's own workgroups nearly fill the GPU, partial sums only cost)
             return ops.gemm_skinny(x, w, k_splits=splits, wide=True)
-    if skinny_ok(x, w):
+    # (the product for the logits, fp32 out over a whole vocabulary: from 9 rows on the library's is the faster one,
+    # 8B shape at 12 / 16 rows 189 / 192 us against 204 / 220)
+    if skinny_ok(x, w) and not (out_dtype == torch.float32 and x.shape[0] > LOGITS_SKINNY_ROWS):
         return ops.gemm_skinny(x, w, out_dtype, wide=False)
     if out_dtype == torch.bfloat16:
         return torch.nn.functional.linear(x, w)
