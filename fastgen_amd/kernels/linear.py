@@ -57,14 +57,22 @@ def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 def fused_gate_up_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """The gate/up product with ``silu(gate) * up`` in its epilogue, where that beats the library's product plus
-    an activation kernel: up to 80 rows (8B shape at 80 rows: 63 us against 64 + 8; at 96 rows 66 against 54 + 8)."""
-    return x.shape[0] <= FUSED_GATE_UP_ROWS and _aligned(x, w)
+    an activation kernel: up to 80 rows (8B shape at 80 rows: 63 us against 64 + 8; at 96 rows 66 against 54 + 8).
+    Above 16 rows only for k below 8,192: the wide kernel streams 4.4 to 4.7 TB/s whatever the size, the library
+    reaches 5.4 on the 70B shape's 939 MB (17 / 64 rows: 174 / 184 us with the activation kernel against 199 / 209)
+    and 3.7 on the 8B shape's 235 MB (65 / 65 us against 48 / 59; 3B shape 42 / 35 against 28 / 32)."""
+    rows = x.shape[0]
+    return (rows <= SKINNY_ROWS or (rows <= FUSED_GATE_UP_ROWS and w.shape[1] < 8192)) and _aligned(x, w)
 
 
 def tall_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Up to 128 rows, for a product whose k range is cut (the o and down projections: the library runs them as
-    32 tiles of 128 columns without a cut, 76 / 24 us at 128 rows of the 8B shape against 46 / 18)."""
-    return x.shape[0] <= TALL_ROWS and _aligned(x, w)
+    32 tiles of 128 columns without a cut, 76 / 24 us at 128 rows of the 8B shape against 46 / 18).  Not for 8,192
+    and more output columns with a k range no longer than that (the 70B shape's o projection: the library's 64
+    tiles take 30 / 33 us at 17 / 64 rows against 35 / 39; its down projection, k = 28,672, stays here: 86 / 111
+    against 91 / 141)."""
+    N, K = w.shape
+    return x.shape[0] <= TALL_ROWS and _aligned(x, w) and (N < 8192 or K > N)
 
 
 _n_cus: Optional[int] = None
