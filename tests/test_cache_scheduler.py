@@ -413,6 +413,56 @@ def test_one_step_behind_gives_the_same_requests(seed):
     s2.cache.check()
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_aborts_at_any_time_lose_nothing(seed):
+    """Requests are aborted at random moments (waiting, mid-prompt, decoding with a sample still pending,
+    preempted) while the scheduler runs a step behind: every request is reported exactly once, an aborted one
+    never runs again, its late sample is still filled in, and every page and slot comes back."""
+    from fastgen_amd.engine.scheduler import PENDING
+
+    rng = random.Random(500 + seed)
+    pages = rng.choice([7, 9, 40])
+    s = mk(cache_pages=pages, page=16, max_batch=rng.choice([2, 4]), budget=rng.choice([8, 24, 100]))
+    reqs = [Request(i, [rng.randrange(50) for _ in range(rng.choice([1, 7, 30, 47]))], max_new=rng.choice([1, 5, 30]),
+                    truncate=True) for i in range(12)]
+    for r in reqs:
+        s.add(r)
+    in_flight, reported, aborted = None, [], set()
+    for _ in range(10_000):
+        reported += [r.rid for r in s.finished]
+        s.finished.clear()
+        if not s.has_work() and in_flight is None:
+            break
+        if rng.random() < 0.3:
+            victim = rng.choice(reqs)
+            if victim.finish_reason is None:
+                assert s.abort(victim.rid)
+                aborted.add(victim.rid)
+            else:
+                assert not s.abort(victim.rid)  # ended already: nothing to abort
+        plan = s.plan()
+        if plan:
+            for e in plan:
+                assert e.request.rid not in aborted and e.request.finish_reason is None
+                s.cache.advance(e.request.rid, e.n)
+            s.cache.check()
+            tokens = [fake_token(e.request, e.start + e.n) for e in plan if e.wants_logits]
+            s.commit(plan)
+        if in_flight is not None:
+            s.resolve(*in_flight)
+            in_flight = None
+        if plan:
+            in_flight = (plan, tokens)
+    else:
+        raise AssertionError("the scheduler did not finish")
+    assert sorted(reported) == list(range(12))
+    for r in reqs:
+        assert r.n_pending == 0 and PENDING not in r.generated
+        assert (r.finish_reason == "aborted") == (r.rid in aborted)
+    assert s.cache.live_requests() == [] and s.cache.free_pages() == pages and s.cache.free_slots() == s.max_batch
+    s.cache.check()
+
+
 def test_a_stop_id_seen_a_step_late_drops_the_step_after_it():
     from fastgen_amd.engine.scheduler import PENDING
 
