@@ -335,6 +335,43 @@ def test_overlap_and_graphs_do_not_change_a_token(dtype, stops, monkeypatch):
         assert run(overlap, graphs) == base, (overlap, graphs)
 
 
+@pytest.mark.parametrize("overlap", [True, False])
+def test_abort_in_the_middle_leaves_the_others_alone(tiny_b, overlap):
+    """A request is aborted while it decodes (with overlapped steps: while its last sample is still on
+    the device), another while it waits: each comes out once, as aborted, with the tokens it had and
+    nothing unresolved among them; the others generate what they generate without them (float32: the
+    plain implementation's tokens); every page comes back."""
+    from fastgen_amd.engine import Engine
+    from fastgen_amd.sampling import SamplingParams
+
+    eng = Engine.from_folder(tiny_b["folder"], torch.float32, page_size=32, max_tokens=1024, max_batch=3,
+                             max_step_tokens=24, overlap_steps=overlap, sync_freq=1)
+    params = SamplingParams(temperature=0.0, max_new_tokens=12)
+    rids = [eng.add_request(p, params) for p in tiny_b["prompts"]]  # five requests, three at a time
+    ended = {}
+    steps = 0
+    while eng.has_work():
+        for r in eng.step():
+            assert r.rid not in ended
+            ended[r.rid] = r
+        steps += 1
+        if steps == 4:
+            assert eng.abort(rids[1])      # decoding by now (a prompt of 12 tokens)
+            assert eng.abort(rids[4])      # still waiting for a place
+            assert not eng.abort("nobody")
+    assert sorted(ended) == sorted(rids)
+    for i in (1, 4):
+        r = ended[rids[i]]
+        assert r.finish_reason == "aborted" and r.n_pending == 0 and all(t >= 0 for t in r.generated)
+    assert 0 < len(ended[rids[1]].generated) < 12 and ended[rids[4]].generated == []
+    assert ended[rids[1]].generated == plain_greedy(tiny_b["weights"], TINY_B, tiny_b["prompts"][1], 12)[: len(ended[rids[1]].generated)]
+    for i in (0, 2, 3):
+        assert ended[rids[i]].finish_reason == "length"
+        assert ended[rids[i]].generated == plain_greedy(tiny_b["weights"], TINY_B, tiny_b["prompts"][i], 12)
+    assert eng.runner.cache.live_requests() == []
+    eng.runner.cache.check()
+
+
 def test_reference_style_interface(tiny_b):
     from fastgen_amd.generate import Fastgen, GenArgs, Packet
 
