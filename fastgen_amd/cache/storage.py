@@ -44,25 +44,49 @@ def bytes_per_token(groups: Sequence[CacheGroup], dtype: torch.dtype) -> int:
     return sum(len(g.entries) * g.need.n_kv_heads * (g.need.head_dim + g.need.value_dim) * esize for g in groups)
 
 
+def state_bytes(state_needs: Dict[int, StateNeed], n_slots: int) -> int:
+    """Bytes of the per-request state tensors for ``n_slots`` slots (and the one row that is nobody's)."""
+    total = 0
+    for need in state_needs.values():
+        n = 1
+        for d in need.shape:
+            n *= int(d)
+        total += (n_slots + 1) * n * torch.empty((), dtype=need.dtype).element_size()
+    return total
+
+
+def tokens_that_fit(free_bytes: int, groups: Sequence[CacheGroup], page_size: int, dtype: torch.dtype,
+                    reserve_bytes: int, state_needs: Optional[Dict[int, StateNeed]] = None, n_slots: int = 0,
+                    at_most: Optional[int] = None) -> int:
+    """Tokens of cache, a whole number of pages, that ``free_bytes`` hold beside ``reserve_bytes`` and the
+    state tensors of ``n_slots`` requests (0: less than one page fits)."""
+    per_token = max(1, bytes_per_token(groups, dtype))
+    left = free_bytes - reserve_bytes - state_bytes(state_needs or {}, n_slots)
+    tokens = max(0, int(left // per_token))
+    if at_most is not None:
+        tokens = min(tokens, at_most)
+    return tokens // page_size * page_size
+
+
 def tokens_for_free_memory(groups: Sequence[CacheGroup], page_size: int, dtype: torch.dtype,
-                           device: torch.device | str, reserve_bytes: int, at_most: Optional[int] = None) -> int:
+                           device: torch.device | str, reserve_bytes: int, at_most: Optional[int] = None,
+                           state_needs: Optional[Dict[int, StateNeed]] = None, n_slots: int = 0) -> int:
     """The cache that the device's free memory holds beside ``reserve_bytes`` (activations of the
-    largest step, captured steps, the libraries' work space), in tokens, a whole number of pages.
+    largest step, captured steps, the libraries' work space) and beside the per-request state of
+    ``n_slots`` requests, in tokens, a whole number of pages.
     The reference sizes its cache from a memory budget the same way (``fastgen/utils/tune.py:68-84``,
     ``fastgen/generate.py:224-238``); here the budget is what the device reports as free now, after
     the weights are in place.  ``at_most``: no more than this many tokens are ever needed."""
     free, _total = torch.cuda.mem_get_info(torch.device(device))
     # what torch's allocator holds but does not use is free for the pools as well
     free += torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
-    per_token = max(1, bytes_per_token(groups, dtype))
-    tokens = int((free - reserve_bytes) // per_token)
-    if at_most is not None:
-        tokens = min(tokens, at_most)
-    tokens = tokens // page_size * page_size
+    tokens = tokens_that_fit(free, groups, page_size, dtype, reserve_bytes, state_needs, n_slots, at_most)
     if tokens < page_size:
+        per_token = max(1, bytes_per_token(groups, dtype))
         raise RuntimeError(
             f"no room for one cache page: {free / 1e9:.2f} GB are free on {device}, {reserve_bytes / 1e9:.2f} GB"
-            f" are kept for the steps' activations, a page of {page_size} tokens takes {per_token * page_size / 1e6:.2f} MB"
+            f" are kept for the steps' activations, {state_bytes(state_needs or {}, n_slots) / 1e9:.2f} GB for the"
+            f" requests' state, a page of {page_size} tokens takes {per_token * page_size / 1e6:.2f} MB"
         )
     return tokens
 

@@ -7,6 +7,7 @@ interface on top of this class.)
 
 from __future__ import annotations
 
+import logging
 import os
 import time
 from dataclasses import dataclass
@@ -20,6 +21,9 @@ from .context import StepEntry
 from .model import Model
 from .runner import ModelRunner
 from .scheduler import PENDING, PlannedEntry, Request, Scheduler
+
+
+logger = logging.getLogger("fastgen_amd")
 
 
 @dataclass
@@ -87,6 +91,7 @@ class Engine:
         self._in_flight: Optional[_InFlight] = None
         self._held: List[Request] = []  # ended, with samples still on the device
         self._n_requests = 0
+        self._logged_running = -1  # the batch size that the log line of the last decode run named
         self.n_steps = 0
         self.last_mean_context = 0.0  # set by time_decode
 
@@ -138,6 +143,9 @@ class Engine:
                 self._settle()  # a decode run starts from tokens the host knows; a stop id among them may end one
             n_run = sched.plan_decode_run(self.sync_freq)
             if n_run:
+                if len(sched.running) != self._logged_running:  # (the reference logs its active lanes so)
+                    self._logged_running = len(sched.running)
+                    logger.info("%d running, decoding %d steps at a time", self._logged_running, n_run)
                 return self._ended(self._decode_run(n_run))
         plan = sched.plan()
         if not plan:
@@ -155,6 +163,11 @@ class Engine:
             entries.append(StepEntry(e.request.rid, toks, [e.n - 1] if e.wants_logits else [], from_row))
             if e.wants_logits:
                 rows.append(e.request)
+        if logger.isEnabledFor(logging.INFO):
+            self._logged_running = -1
+            n_tokens = sum(e.n for e in plan)
+            logger.info("step %d: %d running, %d waiting, %d tokens (%d of prompts)", self.n_steps,
+                        len(sched.running), len(sched.waiting), n_tokens, n_tokens - len(rows))
         logits = self.runner.step(entries, prev.tokens if prev is not None else None)
         self.n_steps += 1
         tok = lps = None

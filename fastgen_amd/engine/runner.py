@@ -10,6 +10,7 @@ is one, because a decoded token is a portion of length one.
 
 from __future__ import annotations
 
+import logging
 import os
 from typing import Dict, Hashable, Optional, Sequence, Tuple
 
@@ -43,6 +44,9 @@ def graph_table_width_for(n_pages: int, limit: int) -> int:
     while w < n_pages:
         w *= 2
     return max(1, min(w, limit))
+
+
+logger = logging.getLogger("fastgen_amd")
 
 
 class _DecodeGraph:
@@ -129,7 +133,8 @@ class ModelRunner:
         self.groups = group_entries(model.paged_needs())
         if max_tokens is None and pages_per_group is None:
             max_tokens = tokens_for_free_memory(self.groups, page_size, model.dtype, model.device, reserve_bytes,
-                                                at_most_tokens) if self.groups else page_size
+                                                at_most_tokens, model.state_needs(), max_requests
+                                                ) if self.groups else page_size
         n_pages = -(-max_tokens // page_size)
         pages = list(pages_per_group) if pages_per_group is not None else [n_pages] * len(self.groups)
         self.cache = CacheManager(page_size, pages, [g.need.window for g in self.groups], max_requests)
@@ -147,6 +152,10 @@ class ModelRunner:
         self.graph_pool = None
         self.graph_capacity = graph_capacity_for  # batch size -> sequences of the recorded step that serves it
         self.max_graphs = 64
+        logger.info("weights %.2f GB; cache %s pages of %d tokens (%.2f GB), %d request slots; decode steps are %s",
+                    model.weight_bytes() / 1e9, pages, page_size,
+                    sum(t.numel() * t.element_size() for t in self.storage.k + self.storage.v) / 1e9, max_requests,
+                    "recorded as graphs" if self.use_graphs else "run eagerly")
         self.run_ahead = 16  # steps the host may prepare before the device has run them
 
     # ------------------------------------------------------------ requests
@@ -236,6 +245,8 @@ class ModelRunner:
                 torch.cuda.synchronize(self.model.device)  # its last replay may still be running
                 self.graphs.pop(next(iter(self.graphs)))
             g = _DecodeGraph(self, entries, key[1])
+            logger.info("recorded a decode step for %d sequences, block tables %d pages wide (%d recorded steps)",
+                        key[0], key[1], len(self.graphs) + 1)
         self.graphs[key] = g  # most recently used last
         return g
 

@@ -14,6 +14,7 @@ from __future__ import annotations
 import logging
 import os
 import queue
+import weakref
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Any, Iterator, List, Optional, Sequence
@@ -21,6 +22,7 @@ from typing import Any, Iterator, List, Optional, Sequence
 import torch
 
 from .engine import Engine, Model
+from .engine.trace_window import TraceWindow
 from .sampling import SamplingParams
 
 logger = logging.getLogger(__name__)
@@ -104,20 +106,42 @@ class HfLoader:
         return FolderTokenizer.maybe(self.model_dir)
 
 
+# The engine that SIGUSR2 asks for a trace: the one built last, held weakly, so that an engine that its
+# owner has dropped gives its memory back and a later one gets the signal.
+_signalled: Optional["weakref.ref[Fastgen]"] = None
+
+
+def _on_profile_signal(_signum, _frame) -> None:
+    fg = _signalled() if _signalled is not None else None
+    if fg is not None:
+        fg.request_profile()
+
+
+def _route_profile_signal_to(fg: "Fastgen", signum: Optional[int] = None) -> None:
+    """SIGUSR2 requests a trace from ``fg``, if nobody else handles that signal
+    (``fastgen/generate.py:165-172``) and this is the main thread (only there can a handler be set)."""
+    import signal
+    import threading
+
+    global _signalled
+    signum = signal.SIGUSR2 if signum is None else signum
+    if threading.current_thread() is not threading.main_thread():
+        return
+    current = signal.getsignal(signum)
+    if current is not signal.SIG_DFL and current is not _on_profile_signal:
+        logger.warning("a handler for signal %s is set; the profile handler was not installed", signum)
+        return
+    _signalled = weakref.ref(fg)
+    if current is signal.SIG_DFL:
+        signal.signal(signum, _on_profile_signal)
+
+
 class Fastgen:
     def __init__(self, engine: Engine, gen_args: GenArgs, stop_tokens: Sequence[int] = ()) -> None:
         self.engine, self.gen_args, self.stop_tokens = engine, gen_args, tuple(stop_tokens)
-        # A trace on request (``fastgen/generate.py:187-196, 364-403``): ``request_profile()``, or the signal
-        # SIGUSR2 where ``build`` could install its handler, starts ``torch.profiler`` at the top of the next
-        # iteration of the generation loop; after FG_PROFILE_ITERS iterations (default 8) a chrome trace is
-        # written to FG_PROFILE_DIR (default /tmp) as fastgen_<pid>_<HHMMSS.f>.json.gz.
-        self.profile_state = "inactive"  # inactive / requested / active
-        self.profile_iter = 0
-        self.profile_iters = int(os.environ.get("FG_PROFILE_ITERS", "8"))
-        self.profile_dir = os.environ.get("FG_PROFILE_DIR", "/tmp")
-        self.last_profile: Optional[str] = None  # the trace written last
-        self._profile_ctx: Any = None
-        self._profile_obj: Any = None
+        # a trace on request: ``request_profile()``, or the signal SIGUSR2 where ``build`` could install
+        # its handler (see ``engine.trace_window``)
+        self.trace = TraceWindow.from_env()
 
     @classmethod
     def build(cls, loader: "HfLoader | str | Path", gen_args: GenArgs = GenArgs(), tp_mesh: Any = None,
@@ -173,60 +197,14 @@ class Fastgen:
                     engine.scheduler.pool_tokens, gen_args.cache_block, engine.scheduler.max_batch)
         engine.runner.max_graphs = max(0, gen_args.num_cuda_graphs)
         fg = cls(engine, gen_args, stop_tokens)
-        fg._install_profile_signal()
+        _route_profile_signal_to(fg)
         return fg
 
     # ---------------------------------------------------------- profiling
-    def _install_profile_signal(self, signum: Optional[int] = None) -> None:
-        """SIGUSR2 requests a trace, if nobody else handles that signal (generate.py:165-172) and this
-        is the main thread (only there can a handler be set)."""
-        import signal
-        import threading
-
-        signum = signal.SIGUSR2 if signum is None else signum
-        if threading.current_thread() is not threading.main_thread():
-            return
-        if signal.getsignal(signum) is not signal.SIG_DFL:
-            logger.warning("a handler for signal %s is set; the profile handler was not installed", signum)
-            return
-        signal.signal(signum, lambda _signum, _frame: self.request_profile())
-
     def request_profile(self) -> None:
-        """Ask for a trace of the next ``FG_PROFILE_ITERS`` iterations of the generation loop."""
-        if self.profile_state == "inactive":
-            logger.info("profile trace requested")
-            self.profile_state = "requested"
-
-    def _profile_step(self) -> None:
-        if self.profile_state == "active":
-            self.profile_iter += 1
-            if self.profile_iter >= self.profile_iters:
-                self._profile_done()
-            return
-        from torch.profiler import ProfilerActivity, profile
-
-        self.profile_iter = 0
-        self._profile_ctx = profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA], with_stack=True)
-        self._profile_obj = self._profile_ctx.__enter__()
-        self.profile_state = "active"
-
-    def _profile_done(self, dump: bool = True) -> None:
-        if self.profile_state != "active":
-            return
-        self.profile_state = "inactive"
-        try:
-            self._profile_ctx.__exit__(None, None, None)
-            if dump:
-                from datetime import datetime
-
-                path = f"{self.profile_dir}/fastgen_{os.getpid()}_{datetime.now().strftime('%H%M%S.%f')}.json.gz"
-                self._profile_obj.export_chrome_trace(path)
-                self.last_profile = path
-                logger.info("profile chrome trace exported to %s", path)
-        except Exception as e:  # a trace that cannot be written must not end the generation
-            logger.warning("error while exporting the profile trace: %r", e)
-        finally:
-            self._profile_ctx = self._profile_obj = None
+        """Ask for a trace of the next ``FG_PROFILE_ITERS`` iterations of the generation loop (the
+        reference's hook of the same name, ``fastgen/generate.py:187-196``)."""
+        self.trace.request()
 
     def _params(self, pkt: Packet) -> SamplingParams:
         ga = self.gen_args
@@ -247,8 +225,7 @@ class Fastgen:
         pending = {}
         refused: List[Packet] = []
         while True:
-            if self.profile_state != "inactive":
-                self._profile_step()
+            self.trace.tick()
             while not eoq:
                 try:
                     pkt = q.get(block=not self.engine.has_work())
@@ -271,7 +248,7 @@ class Fastgen:
                 yield refused.pop(0)
             if not self.engine.has_work():
                 if eoq:
-                    self._profile_done()  # a trace that was still running is written with what it has
+                    self.trace.close()  # a trace that was still running is written with what it has
                     return
                 continue
             for req in self.engine.step():

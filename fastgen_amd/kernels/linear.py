@@ -1,18 +1,21 @@
 """``y = x W^T`` for the two precisions of the engine.
 
 float32: the engine's own fused-multiply-add kernel (``gemm.hip``), a true
-32-bit product whose rows do not depend on one another.  bfloat16: up to 16
-rows (decode) the engine's weight-streaming MFMA kernel (``gemm_skinny.hip``);
-up to 64 rows (128 where the k range is cut) its wider sibling where that beats
-the library; otherwise the vendor library's matrix product through ``torch`` (the
-reference uses cuBLAS through ``F.linear`` for all of them,
-``fastgen/forward.py:433-513``), with fp32 accumulation; logits are asked for in
-fp32 directly.
+32-bit product whose rows do not depend on one another.  bfloat16: several
+kernels can take a product (the engine's weight-streaming MFMA kernels of
+``gemm_skinny.hip``, narrow and wide, with or without a cut of the k range, and
+the vendor library's product through ``torch``, which the reference uses for
+all of them: cuBLAS through ``F.linear``, ``fastgen/forward.py:433-513``).
+Which one is the fastest depends on the matrix and on the number of rows, so
+it is measured: the first time a product of some shape ``(N, K)`` meets some
+number of rows, the kernels that can take it are timed on the operands at hand
+and the winner is kept in one table (``choices``) for every later product of
+that shape and row bucket.  No size of any model stands here or in the parts.
 """
 
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
 
@@ -37,11 +40,9 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
         raise
 
 
-# up to this many rows the weight-streaming kernels are used (more: the library's product)
-SKINNY_ROWS = 16  # one 16-row block of x, 16 output columns a workgroup
-FUSED_GATE_UP_ROWS = 80
-LOGITS_SKINNY_ROWS = 8
-TALL_ROWS = 128   # with k splits (few output columns, long k) the same kernel with up to eight blocks of x
+# what the kernels take (their limits, not a model's sizes)
+SKINNY_ROWS = 16  # one 16-row block of x: the narrow kernel (16 output columns a workgroup) and every folded epilogue
+WIDE_ROWS = ops.SKINNY_MAX_ROWS  # the wide kernel (64 columns a workgroup): up to eight blocks of x
 
 
 def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -51,46 +52,9 @@ def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Few rows (decode): the engine's own weight-streaming kernel takes the product."""
+    """Few rows (decode): the engine's own weight-streaming kernels take the product, with the
+    epilogues that are folded into them."""
     return x.shape[0] <= SKINNY_ROWS and _aligned(x, w)
-
-
-def fused_gate_up_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """The gate/up product with ``silu(gate) * up`` in its epilogue, where that beats the library's product plus
-    an activation kernel: up to 80 rows (8B shape at 80 rows: 63 us against 64 + 8; at 96 rows 66 against 54 + 8).
-    Above 16 rows only for k below 8,192: the wide kernel streams 4.4 to 4.7 TB/s whatever the size, the library
-    reaches 5.4 on the 70B shape's 939 MB (17 / 64 rows: 174 / 184 us with the activation kernel against 199 / 209)
-    and 3.7 on the 8B shape's 235 MB (65 / 65 us against 48 / 59; 3B shape 42 / 35 against 28 / 32)."""
-    rows = x.shape[0]
-    return (rows <= SKINNY_ROWS or (rows <= FUSED_GATE_UP_ROWS and w.shape[1] < 8192)) and _aligned(x, w)
-
-
-def tall_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Up to 128 rows, for a product whose k range is cut (the o and down projections: the library runs them as
-    32 tiles of 128 columns without a cut, 76 / 24 us at 128 rows of the 8B shape against 46 / 18).  Not for 8,192
-    and more output columns with a k range no longer than that (the 70B shape's o projection: the library's 64
-    tiles take 30 / 33 us at 17 / 64 rows against 35 / 39; its down projection, k = 28,672, stays here: 86 / 111
-    against 91 / 141)."""
-    N, K = w.shape
-    return x.shape[0] <= TALL_ROWS and _aligned(x, w) and (N < 8192 or K > N)
-
-
-_n_cus: Optional[int] = None
-
-
-def _compute_units() -> int:
-    global _n_cus
-    if _n_cus is None:
-        _n_cus = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
-    return _n_cus
-
-
-def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
-    """Splits of the k range that give the wide kernel (64 output columns a workgroup) about two
-    workgroups per compute unit, at most 8; with many rows a split keeps at least 1,024 of k (the
-    partial sums it writes grow with the rows), else 512.  1: the output is wide enough by itself."""
-    blocks = -(-n_out // 64)
-    return max(1, min(8, 2 * _compute_units() // blocks, k // (1024 if rows > 48 else 512)))
 
 
 def fold_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -99,49 +63,141 @@ def fold_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
     return skinny_ok(x, w)
 
 
+def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
+    """Splits of the k range that give the wide kernel (64 output columns a workgroup) about two
+    workgroups per compute unit, at most 8; with many rows a split keeps at least 1,024 of k (the
+    partial sums it writes grow with the rows), else 512.  1: the output is wide enough by itself."""
+    blocks = -(-n_out // 64)
+    return max(1, min(8, 2 * ops.compute_units() // blocks, k // (1024 if rows > 48 else 512)))
+
+
+# ------------------------------------------------------------------ the table
+# (what is asked for, N, K, row bucket) -> name of the kernel that measured fastest
+choices: Dict[Tuple[str, int, int, int], str] = {}
+# set to a candidate's name to take that kernel wherever it is among the candidates (tests run the
+# engine once under each name, so that every kernel that may be chosen is compared with the plain run)
+force: Optional[str] = None
+_TIMED_RUNS = 4
+
+
+def row_bucket(rows: int) -> int:
+    """Products of up to 16 rows are measured per number of rows, above that per block of 16 rows
+    (the kernels work on such blocks), above the widest own kernel as one."""
+    if rows <= SKINNY_ROWS:
+        return rows
+    return min(-(-rows // 16) * 16, WIDE_ROWS + 16)
+
+
+def _capturing() -> bool:
+    return torch.cuda.is_current_stream_capturing()
+
+
+def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Callable[[], torch.Tensor]]]) -> str:
+    """The candidate to run: the forced one, the one the table holds, or the one that is fastest now.
+    Timing needs the device to itself (events and a wait for them), so a product that is first met while
+    a step is being recorded runs the first candidate, unrecorded in the table; the engine runs every
+    step once, unrecorded, before it records it.  The candidates are timed in turn on the same
+    operands, each run behind a run of the other."""
+    names = [c[0] for c in candidates]
+    if force in names:
+        return force
+    if len(candidates) == 1:
+        return names[0]
+    key = (what, n, k, row_bucket(rows))
+    got = choices.get(key)
+    if got in names:
+        return got
+    if _capturing():
+        return names[0]
+    best: Dict[str, float] = {}
+    for fn in (c[1] for c in candidates):  # once each, unmeasured: libraries load, the library picks its kernel
+        fn()
+    events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+               for _ in range(_TIMED_RUNS)] for _ in candidates]
+    for r in range(_TIMED_RUNS):
+        for ev, (_, fn) in zip(events, candidates):
+            ev[r][0].record()
+            fn()
+            ev[r][1].record()
+    torch.cuda.current_stream().synchronize()
+    for ev, name in zip(events, names):
+        best[name] = min(a.elapsed_time(b) for a, b in ev)
+    winner = min(names, key=lambda nm: best[nm])
+    choices[key] = winner
+    return winner
+
+
 def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           partials_ok: bool = False, residual: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None):
+           partials_ok: bool = False, residual: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None,
+           epilogue: Optional[str] = None):
     """``x @ w.T``.  With ``partials_ok`` the result may come as fp32 ``[S, M, N]``
     partial sums whose sum over ``S`` is the product (the caller hands it to a
     norm, which adds them in order).
+
+    ``epilogue="silu_mul"``: ``w`` is a gate and an up matrix interleaved by
+    :func:`~fastgen_amd.kernels.ops.interleave_gate_up` and the result is
+    ``silu(gate) * up`` ``[M, N/2]``, in the product's kernel where one that does so is the fastest.
 
     ``x`` may be :class:`~fastgen_amd.kernels.ops.ScaledRows`.  ``residual`` = (h, norm weight,
     eps) asks for more than the product: add it to the fp32 residual stream ``h`` and prepare the
     RMSNorm that follows.  Where that can be folded into the product's kernel (few rows, bfloat16)
     the result is ``ScaledRows`` and ``h`` is updated; where not, the plain product comes back and
     adding and norming are the caller's."""
+    silu = epilogue == "silu_mul"
+    if epilogue not in (None, "silu_mul"):
+        raise ops.KernelArgumentError(f"linear: unknown epilogue {epilogue!r}")
     scaled = x if isinstance(x, ops.ScaledRows) else None
     if scaled is not None:
-        if not fold_ok(scaled.rows, w):
+        if not fold_ok(scaled.rows, w) or out_dtype not in (None, torch.bfloat16):
             x, scaled = scaled.materialize(), None
         else:
             x = scaled.rows
-    if residual is not None and x.is_cuda and fold_ok(x, w) and out_dtype in (None, torch.bfloat16):
-        h, norm_w, eps = residual
-        if h.dtype == torch.float32 and h.is_contiguous() and h.shape == (x.shape[0], w.shape[0]):
-            return ops.gemm_skinny_residual(scaled or x, w, h, norm_w, eps)
-    if scaled is not None:
-        if out_dtype in (None, torch.bfloat16):
-            return ops.gemm_skinny(scaled, w, torch.bfloat16, wide=False)
-        x = scaled.materialize()
     if not x.is_cuda:
         raise ops.KernelArgumentError("fastgen_amd runs on the GPU only; got a tensor on " + str(x.device))
-    out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
-        if out_dtype != torch.float32:
+        if out_dtype not in (None, torch.float32):
             raise ops.KernelArgumentError("a float32 product has float32 output")
-        return ops.gemm_nt(x, w)
+        y = ops.gemm_nt(x, w)
+        return ops.silu_mul(y) if silu else y
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise ops.KernelArgumentError(f"linear: unsupported dtypes {x.dtype}, {w.dtype}")
-    if partials_ok and x.shape[0] > 2 and tall_ok(x, w):
-        splits = k_splits_for(w.shape[0], w.shape[1], x.shape[0])
-        if splits > 3:  # (fewer: the output's own workgroups nearly fill the GPU, partial sums only cost)
-            return ops.gemm_skinny(x, w, k_splits=splits, wide=True)
-    # (the product for the logits, fp32 out over a whole vocabulary: from 9 rows on the library's is the faster one,
-    # 8B shape at 12 / 16 rows 189 / 192 us against 204 / 220)
-    if skinny_ok(x, w) and not (out_dtype == torch.float32 and x.shape[0] > LOGITS_SKINNY_ROWS):
-        return ops.gemm_skinny(x, w, out_dtype, wide=False)
-    if out_dtype == torch.bfloat16:
-        return torch.nn.functional.linear(x, w)
-    y = _library_mm_f32_out(x, w)
-    return y if y is not None else ops.gemm_nt(x, w, out_dtype=torch.float32)
+    out_dtype = out_dtype or torch.bfloat16
+    rows, (N, K) = x.shape[0], w.shape
+    own = _aligned(x, w)
+    src = scaled or x  # what the own kernels are given: they finish a norm that is still open
+
+    if residual is not None and own and rows <= SKINNY_ROWS and out_dtype == torch.bfloat16 and not silu:
+        h, norm_w, eps = residual
+        if h.dtype == torch.float32 and h.is_contiguous() and h.shape == (rows, N):
+            return ops.gemm_skinny_residual(src, w, h, norm_w, eps)
+
+    def library() -> torch.Tensor:
+        xin = scaled.materialize() if scaled is not None else x
+        if out_dtype == torch.bfloat16:
+            y = torch.nn.functional.linear(xin, w)
+        else:
+            y = _library_mm_f32_out(xin, w)
+            if y is None:
+                y = ops.gemm_nt(xin, w, out_dtype=torch.float32)
+        return ops.silu_mul(y) if silu else y
+
+    candidates: List[Tuple[str, Callable[[], torch.Tensor]]] = []
+    if own and silu and out_dtype == torch.bfloat16 and N % 16 == 0:
+        if rows <= SKINNY_ROWS:
+            candidates.append(("narrow", lambda: ops.gemm_skinny(src, w, silu_mul_epilogue=True, wide=False)))
+        if rows <= WIDE_ROWS:
+            candidates.append(("wide", lambda: ops.gemm_skinny(src, w, silu_mul_epilogue=True, wide=True)))
+    elif own and not silu:
+        if rows <= SKINNY_ROWS:
+            candidates.append(("narrow", lambda: ops.gemm_skinny(src, w, out_dtype, wide=False)))
+        elif rows <= WIDE_ROWS and partials_ok:
+            splits = k_splits_for(N, K, rows)
+            candidates.append(("wide", lambda: ops.gemm_skinny(x, w, out_dtype, k_splits=splits, wide=True)))
+        elif rows <= 64:
+            candidates.append(("wide", lambda: ops.gemm_skinny(x, w, out_dtype, wide=True)))
+    if scaled is None or not candidates:
+        candidates.append(("library", library))
+    what = ("silu_mul" if silu else "store") + ("+partials" if partials_ok and rows > SKINNY_ROWS else "") + (
+        "+f32" if out_dtype == torch.float32 else "") + ("+scaled" if scaled is not None else "")
+    name = _choose(what, N, K, rows, candidates)
+    return dict(candidates)[name]()

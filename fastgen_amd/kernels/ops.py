@@ -268,11 +268,26 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
 
 MFMA_MAX_HEAD_DIM = 256
 
-# Workgroups wanted for the decode attention kernel: one per CU measured best (256 CUs; 128 to 2048
-# tried at batch 1, 8 and 64).  The splits' partial results are merged by a second kernel: merging
-# them in the split that finishes last needs device-scope fences, which on a GPU of several
-# dies cost more than the launch they save (measured).
-_SPLIT_TARGET_BLOCKS = int(os.environ.get("FG_SPLIT_TARGET", 256))
+_n_cus: Optional[int] = None
+
+
+def compute_units() -> int:
+    """Compute units of the current device (asked once)."""
+    global _n_cus
+    if _n_cus is None:
+        _n_cus = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+    return _n_cus
+
+
+def _split_target_blocks() -> int:
+    """Workgroups wanted for the decode attention kernel: one per compute unit measured best (half as many
+    to eight times as many tried at batch 1, 8 and 64).  The splits' partial results are merged by a second
+    kernel: merging them in the split that finishes last needs device-scope fences, which on a GPU of
+    several dies cost more than the launch they save (measured)."""
+    env = os.environ.get("FG_SPLIT_TARGET")
+    return int(env) if env else compute_units()
+
+
 # a chunk of the decode attention's key ranges is a multiple of this many 64-key tiles (one a wave)
 _SPLIT_MIN_TILES = int(os.environ.get("FG_SPLIT_MIN_TILES", 4))
 
@@ -309,7 +324,7 @@ def attention_chunks_for(n_items: int, n_kv: int) -> int:
     """Length of the split kernel's chunk list for ``n_items`` items: enough chunks for a few
     workgroups per compute unit, and at least two an item so that a long sequence among short
     ones can be cut."""
-    return max(-(-_SPLIT_TARGET_BLOCKS // n_kv) + n_items, 2 * n_items)
+    return max(-(-_split_target_blocks() // n_kv) + n_items, 2 * n_items)
 
 
 def _plan_ints(lib, max_chunks: int) -> int:

@@ -1,7 +1,7 @@
 """A plain PyTorch function beside every kernel of ``ops``: the same name, the
 same arguments, the same effect on the same tensors, written as the formula
 and not as the kernel works.  They say what each kernel computes and are what
-the kernels are held to in ``tests/test_gpu_twins.py``; nothing of the engine
+the kernels are held to in ``tests/test_twins.py``; nothing of the engine
 calls them (the engine has no execution path but its kernels), and they work
 on CPU tensors as well as on GPU ones.
 

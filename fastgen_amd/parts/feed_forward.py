@@ -11,7 +11,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import fused_gate_up_ok, linear, skinny_ok
+from ..kernels.linear import linear
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
@@ -48,19 +48,7 @@ class SwiGLU(FeedForward):
     def forward(self, x, then=None):
         """``x``: the normed rows, or ``ScaledRows`` (the gate/up product finishes the norm).  ``then``:
         a norm's ``fold_request`` for the down projection (see ``Attention.forward``)."""
-        rows = x.rows if isinstance(x, ops.ScaledRows) else x
-        if rows is not x and not skinny_ok(rows, self.w_gate_up):
-            x = rows = x.materialize()
-        if fused_gate_up_ok(rows, self.w_gate_up):
-            # From 11 rows on the wide kernel (64 columns a workgroup, x through LDS) is the faster one at the 8B
-            # shape (a decode step of 12 / 14 / 16 sequences 4.60 / 4.71 / 4.80 ms against 4.67 / 4.84 / 5.00; equal
-            # at 10, slower at 9).  Not at the 3B shape (k = 3,072: the wide kernel's 12 passes of loads, one
-            # after the other, take 26 us whatever the rows, the narrow one 24 at 12 rows) nor at the 70B shape
-            # (k = 8,192: 194 us against 182 at 12 rows, equal at 16).
-            wide = rows.shape[0] > 16 or (rows.shape[0] > 10 and 4096 <= self.dim < 8192)
-            act = ops.gemm_skinny(x, self.w_gate_up, silu_mul_epilogue=True, wide=wide)
-        else:
-            act = ops.silu_mul(linear(x, self.w_gate_up))
+        act = linear(x, self.w_gate_up, epilogue="silu_mul")
         return linear(act, self.w_down, partials_ok=True, residual=then)
 
 

@@ -125,23 +125,56 @@ def main(argv: Optional[List[str]] = None) -> int:
         print("fgchat: a dialogue needs tokenizer.json in the model folder; use --prompt-ids or --random-prompt",
               file=sys.stderr)
         return 2
+    print("Commands: /r <N> go back to before round N; /m a message of several lines, ended by a line"
+          " that holds only '.'; /q quit", file=sys.stderr)
+    return dialogue_loop(tokenizer, run)
+
+
+def read_turn(dialog: List[dict], read=input) -> Optional[str]:
+    """One turn of the dialogue's prompt (``fastgen/tools/chat.py:170-195``): returns the user's message, or
+    None when the loop should ask again (a command was carried out); raises EOFError to quit.  ``/r <N>`` cuts
+    the dialogue back to before round N (a round is a user message and its answer), ``/r`` alone drops the last
+    round; ``/m`` reads lines until one that is a single '.'; ``/q`` quits."""
+    n_round = 1 + len(dialog) // 2
+    line = read(f"{n_round}> ").strip()
+    word, _, rest = line.partition(" ")
+    if word == "/q":
+        raise EOFError
+    if word == "/r":
+        try:
+            n = int(rest) if rest.strip() else n_round - 1
+            if n < 1:
+                raise ValueError
+            del dialog[2 * (n - 1):]
+        except ValueError:
+            print("invalid command", file=sys.stderr)
+        return None
+    if word == "/m" and not rest.strip():
+        lines: List[str] = []
+        while True:
+            more = read(f"{n_round}>> ")
+            if more.strip() == ".":
+                break
+            lines.append(more)
+        return "\n".join(lines)
+    return line
+
+
+def dialogue_loop(tokenizer, run, read=input, write=print) -> int:
     dialog: List[dict] = []
     while True:
         try:
-            line = input("> ")
+            msg = read_turn(dialog, read)
         except EOFError:
             return 0
-        if line.strip() == "/q":
-            return 0
-        if line.strip() == "/r":
-            dialog = dialog[:-2]
+        if msg is None:
             continue
-        dialog.append({"role": "user", "content": line})
+        dialog.append({"role": "user", "content": msg})
         out = run(tokenizer.encode_dialog(dialog))
         if out and out[-1] in tokenizer.stop_tokens:
             out = out[:-1]  # tools/chat.py:205-206
         text = tokenizer.decode(out)
-        print(text)
+        write(text)
         dialog.append({"role": "assistant", "content": text})
 
 

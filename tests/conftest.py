@@ -20,3 +20,13 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How much of its tolerance the engine used at most, per precision (tests/helpers.py:assert_close)."""
+    try:
+        from helpers import worst_share
+    except ImportError:
+        return
+    for dtype, (share, what) in sorted(worst_share.items()):
+        terminalreporter.write_line(f"largest share of the {dtype} tolerance used: {share:.3f} ({what})")

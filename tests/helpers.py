@@ -53,15 +53,27 @@ def plain_logits(weights, config, tokens: Mapping[str, List[int]], dtype=torch.f
     return {rid: plain_forward(weights, config, t, dtype) for rid, t in tokens.items()}
 
 
+# the largest share of its tolerance that any comparison of this session has used, per precision
+# (printed when the session ends: a creeping error shows here before it fails a test)
+worst_share: Dict[str, tuple] = {}
+
+# bfloat16: the share of the tolerance below that the engine may use.  The tolerance is twice the plain
+# bfloat16 run's worst error over the request; the most that the engine has been seen to use of it, over all
+# configurations and cuts, is 0.73 (portions of changing size at the smallest configuration), and what a
+# session used at most is printed at its end.
+BF16_SHARE = 0.9
+
+
 def assert_close(got: Mapping[str, torch.Tensor], want: Mapping[str, torch.Tensor], dtype: torch.dtype,
-                 noise: Optional[Mapping[str, torch.Tensor]] = None, what: str = "") -> None:
-    """float32: the engine and the plain implementation differ by rounding of
+                 noise: Optional[Mapping[str, torch.Tensor]] = None, what: str = "") -> float:
+    """Returns the largest share of the tolerance that a position used.  float32: the engine and the plain implementation differ by rounding of
     fp32 sums only: 2e-5 of the largest logit; or, when ``want`` is a float64
     run and ``noise`` the plain float32 run (layers wide enough for the
     rounding of long sums to show), three times what the plain float32 run is
     off.  bfloat16: ``noise`` is the plain implementation run in bfloat16; the
     engine may be off the fp32 result by twice what that run is off, and no
     more."""
+    share = 0.0
     for rid, w in want.items():
         g = got[rid]
         assert g.shape == w.shape, f"{what} {rid}: shape {tuple(g.shape)} vs {tuple(w.shape)}"
@@ -75,11 +87,18 @@ def assert_close(got: Mapping[str, torch.Tensor], want: Mapping[str, torch.Tenso
             tol = 2e-5 * scale
         else:
             tol = 2.0 * float((noise[rid] - w).abs().max()) + 1e-3 * scale
+            tol *= BF16_SHARE
         worst = int(err.argmax())
         assert float(err.max()) <= tol, (
             f"{what} request {rid}: first position over tolerance is "
             f"{int((err > tol).nonzero()[0])} of {len(err)}, worst {worst}: {float(err.max()):.3e} > {tol:.3e}"
+            f" ({float(err.max()) / tol:.2f} of it)"
         )
+        share = max(share, float(err.max()) / tol)
+    key = str(dtype).replace("torch.", "")
+    if share > worst_share.get(key, (0.0, ""))[0]:
+        worst_share[key] = (share, what)
+    return share
 
 
 def write_tiny_tokenizer(folder: Path, n_words: int = 40) -> List[str]:

@@ -378,8 +378,9 @@ def drive_one_step_behind(sched, max_steps=10_000):
     return reported
 
 
+@pytest.mark.parametrize("admit_reserve", [0, 16, 128])
 @pytest.mark.parametrize("seed", range(16))
-def test_one_step_behind_gives_the_same_requests(seed):
+def test_one_step_behind_gives_the_same_requests(seed, admit_reserve):
     """Random loads with stop ids, small budgets and few pages (preemption): every request ends with the
     same tokens and for the same reason whether the scheduler sees a step's tokens at once or a step
     late; nothing is left pending, no page is lost."""
@@ -388,7 +389,7 @@ def test_one_step_behind_gives_the_same_requests(seed):
         # odd seeds: pools so tight that decoding requests are preempted with a sample still pending
         pages = rng.choice([8, 12, 40]) if seed % 2 == 0 else rng.choice([7, 8, 9])
         s = mk(cache_pages=pages, page=16, max_batch=rng.choice([2, 4, 8]),
-               budget=rng.choice([8, 24, 100]), max_seq=rng.choice([None, 60]))
+               budget=rng.choice([8, 24, 100]), max_seq=rng.choice([None, 60]), admit_reserve=admit_reserve)
         reqs = []
         for i in range(14):
             n = rng.choice([1, 3, 20, 45, 90]) if seed % 2 == 0 else rng.choice([7, 15, 30, 31, 47])
@@ -413,8 +414,9 @@ def test_one_step_behind_gives_the_same_requests(seed):
     s2.cache.check()
 
 
+@pytest.mark.parametrize("admit_reserve", [0, 16, 128])
 @pytest.mark.parametrize("seed", range(8))
-def test_aborts_at_any_time_lose_nothing(seed):
+def test_aborts_at_any_time_lose_nothing(seed, admit_reserve):
     """Requests are aborted at random moments (waiting, mid-prompt, decoding with a sample still pending,
     preempted) while the scheduler runs a step behind: every request is reported exactly once, an aborted one
     never runs again, its late sample is still filled in, and every page and slot comes back."""
@@ -422,7 +424,8 @@ def test_aborts_at_any_time_lose_nothing(seed):
 
     rng = random.Random(500 + seed)
     pages = rng.choice([7, 9, 40])
-    s = mk(cache_pages=pages, page=16, max_batch=rng.choice([2, 4]), budget=rng.choice([8, 24, 100]))
+    s = mk(cache_pages=pages, page=16, max_batch=rng.choice([2, 4]), budget=rng.choice([8, 24, 100]),
+           admit_reserve=admit_reserve)
     reqs = [Request(i, [rng.randrange(50) for _ in range(rng.choice([1, 7, 30, 47]))], max_new=rng.choice([1, 5, 30]),
                     truncate=True) for i in range(12)]
     for r in reqs:
@@ -590,3 +593,28 @@ def test_admission_keeps_room_for_what_running_requests_will_generate():
     s3 = mk(cache_pages=2, page=16, max_batch=2, budget=64, admit_reserve=128)
     s3.add(Request("a", [1] * 20, max_new=12))
     assert [e.request.rid for e in s3.plan()] == ["a"]
+
+
+def test_memory_budget_counts_the_per_request_state():
+    """The cache's size from a memory budget: pages take what the reserve and the per-request state
+    tensors (one row a slot, and one more) leave."""
+    import torch
+
+    from fastgen_amd.cache.storage import bytes_per_token, group_entries, state_bytes, tokens_that_fit
+    from fastgen_amd.parts import PagedNeed, StateNeed
+
+    groups = group_entries([PagedNeed(2, 16, None), PagedNeed(2, 16, None), None, PagedNeed(1, 32, 64)])
+    per_token = bytes_per_token(groups, torch.bfloat16)
+    assert per_token == 2 * 2 * 32 * 2 + 1 * 64 * 2
+    needs = {2: StateNeed((100, 8), torch.float32), 3: StateNeed((7,), torch.bfloat16)}
+    assert state_bytes(needs, 9) == 10 * (100 * 8 * 4 + 7 * 2)
+    assert state_bytes({}, 9) == 0
+    free, reserve, page = 10_000_000, 1_000_000, 16
+    plain = tokens_that_fit(free, groups, page, torch.bfloat16, reserve)
+    assert plain == (free - reserve) // per_token // page * page
+    with_state = tokens_that_fit(free, groups, page, torch.bfloat16, reserve, needs, 999)
+    assert with_state == (free - reserve - state_bytes(needs, 999)) // per_token // page * page < plain
+    # the pools and the state together stay inside the budget
+    assert with_state * per_token + state_bytes(needs, 999) + reserve <= free
+    assert tokens_that_fit(free, groups, page, torch.bfloat16, reserve, needs, 999, at_most=100) == 96
+    assert tokens_that_fit(free, groups, page, torch.bfloat16, reserve, needs, 10 ** 6) == 0  # the state alone is too much

@@ -219,3 +219,64 @@ def test_folder_tokenizer(tmp_path):
     want = "<user> w1 w2 <end> <bot> w5 <end> <user> w7 <end> <bot>".split()
     assert tok.encode_dialog(dialog) == [words.index(w) for w in want]
 
+
+
+def test_trace_window_counts_iterations(tmp_path):
+    """A trace on request covers the next ``n_iters`` iterations of the loop that ticks it, is written
+    once, and a second request while one waits or runs is ignored."""
+    from fastgen_amd.engine.trace_window import TraceWindow
+
+    w = TraceWindow(2, str(tmp_path), prefix="t")
+    w.tick()
+    assert not w.pending and not w.recording and w.last_path is None
+    w.request()
+    w.request()
+    assert w.pending and not w.recording
+    w.tick()  # iteration 1 begins
+    assert w.recording and not w.pending
+    w.request()  # ignored: one is running
+    assert not w.pending
+    w.tick()  # iteration 2 begins
+    assert w.recording
+    w.tick()  # both are over
+    assert not w.recording and w.last_path is not None
+    assert [p.name for p in tmp_path.iterdir()] == [w.last_path.rsplit("/", 1)[1]]
+    w.request()
+    w.tick()
+    w.close(write=False)  # a loop that ends early and wants no file
+    assert not w.recording and len(list(tmp_path.iterdir())) == 1
+
+
+def test_chat_dialogue_commands():
+    """The dialogue loop's commands as in ``fastgen/tools/chat.py:161-195``: ``/r <N>`` resets the
+    conversation to before round N, ``/m`` takes a message of several lines, ``/q`` quits."""
+    from fastgen_amd.tools.chat import dialogue_loop
+
+    class Tok:
+        stop_tokens = (99,)
+
+        def encode_dialog(self, dialog):
+            return [len(dialog)] + [len(m["content"]) for m in dialog]
+
+        def decode(self, ids):
+            return "answer to " + ",".join(map(str, ids))
+
+    seen, said = [], []
+    script = iter(["hello", "more", "/r 2", "again", "/m", "line one", "line two", ".", "/r x", "/r", "last", "/q", "never"])
+    prompts = []
+
+    def read(prompt):
+        prompts.append(prompt)
+        return next(script)
+
+    def run(tokens):
+        seen.append(list(tokens))
+        return [len(seen), 99]  # ends on a stop token, which is dropped from the text
+
+    assert dialogue_loop(Tok(), run, read, said.append) == 0
+    # round 1, round 2, back to before round 2, round 2 again, round 3 of two lines, a bad command,
+    # /r alone drops round 3, round 3 again
+    assert [t[0] for t in seen] == [1, 3, 3, 5, 5]
+    assert seen[3][-1] == len("line one\nline two") and seen[2][-1] == len("again")
+    assert said == ["answer to 1", "answer to 2", "answer to 3", "answer to 4", "answer to 5"]
+    assert prompts[:3] == ["1> ", "2> ", "3> "] and "3>> " in prompts and prompts[-1] == "4> "

@@ -45,11 +45,14 @@ def test_greedy_generation_matches_the_plain_implementation(tiny_b):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_decode_batches_between_the_captured_sizes(tiny_b, dtype):
+def test_decode_batches_between_the_captured_sizes(tiny_b, dtype, monkeypatch):
     """21 requests of different lengths decode together and end one after the
     other: batches of 21, 20, ... run on captured steps of 24 and fewer
-    sequences filled up with stand-ins.  Each request's tokens are those it
-    gets alone (float32: those of the plain implementation)."""
+    sequences filled up with stand-ins.  float32: each request's tokens are those
+    of the plain implementation.  bfloat16: an engine-against-engine check, the
+    captured steps against the same engine stepped eagerly (the comparison of this
+    path with the plain implementation is
+    ``test_gpu_engine.py::test_many_requests_decode_together_bfloat16``)."""
     from fastgen_amd.engine import Engine
     from fastgen_amd.engine.runner import graph_capacity_for
     from fastgen_amd.sampling import SamplingParams
@@ -70,15 +73,11 @@ def test_decode_batches_between_the_captured_sizes(tiny_b, dtype):
     else:
         # bfloat16 rounding differs between kernels for few and for many rows: the same engine with
         # the same batches, stepped eagerly, is what the captured steps must reproduce
-        import os
-        os.environ["FG_NO_GRAPHS"] = "1"
-        try:
-            eager = Engine.from_folder(tiny_b["folder"], dtype, page_size=16, max_tokens=21 * 96, max_batch=32,
-                                       max_step_tokens=256)
-            assert not eager.runner.use_graphs
-            want = eager.generate(prompts, params)
-        finally:
-            del os.environ["FG_NO_GRAPHS"]
+        monkeypatch.setenv("FG_NO_GRAPHS", "1")
+        eager = Engine.from_folder(tiny_b["folder"], dtype, page_size=16, max_tokens=21 * 96, max_batch=32,
+                                   max_step_tokens=256)
+        assert not eager.runner.use_graphs
+        want = eager.generate(prompts, params)
         assert got == want
     assert eng.runner.cache.live_requests() == []
     eng.runner.cache.check()
@@ -447,10 +446,16 @@ def test_command_line_with_a_tokenizer(tiny_b, tmp_path):
     assert [int(x) for x in lines[0].split(",")] == want
     assert lines[1] == tok.decode([t for t in want if t != stop])
     # the dialogue loop: the first answer is the same generation
-    proc = subprocess.run(base, input="w1 w2 w3\n/r\nw1 w2 w3\n/q\n", capture_output=True, text=True, timeout=300)
+    # (the prompts "1> ", "2> " of the rounds stand in front of what follows them on stdout), then a reset to
+    # before round 1 and the same message in several lines' form
+    import re
+
+    proc = subprocess.run(base, input="w1 w2 w3\n/r 1\n/m\nw1 w2 w3\n.\n/q\n", capture_output=True, text=True,
+                          timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
-    answers = [l.replace("> ", "") for l in proc.stdout.splitlines() if l.replace("> ", "").strip()]
+    answers = [a for a in (re.sub(r"\d+>+ ", "", l).strip() for l in proc.stdout.splitlines()) if a]
     assert len(answers) == 2 and answers[0] == answers[1] == lines[1]
+    assert "1> " in proc.stdout and "1>> " in proc.stdout and "2> " in proc.stdout
 
 
 def test_smoke_entry():
@@ -615,21 +620,23 @@ def test_profile_trace_on_request(tiny_b, tmp_path, monkeypatch):
     try:
         fg = Fastgen.build(tiny_b["folder"], GenArgs(use_sampling=False, max_batch=2, max_seq=512, max_gen=12,
                                                     cache_block=32, dtype=torch.bfloat16, sync_freq=2), stop_tokens=())
-        assert fg.profile_iters == 3 and fg.profile_state == "inactive"
-        if old is signal.SIG_DFL:  # nobody else handled it: the signal asks for a trace
-            os.kill(os.getpid(), signal.SIGUSR2)
+        assert fg.trace.n_iters == 3 and not fg.trace.pending and not fg.trace.recording
+        from fastgen_amd import generate as generate_module
+
+        if old is signal.SIG_DFL or old is generate_module._on_profile_signal:
+            os.kill(os.getpid(), signal.SIGUSR2)  # nobody else handles it: the signal asks the engine built last
         else:
             fg.request_profile()
-        assert fg.profile_state == "requested"
+        assert fg.trace.pending
         q = queue.Queue()
         for i in (1, 2):
             q.put(Packet(thread_id=i, tokens=tiny_b["prompts"][i]))
         q.put(None)
         out = {p.thread_id: p.tokens for p in fg.generate(q)}
         assert len(out[1]) == len(out[2]) == 12
-        assert fg.profile_state == "inactive" and fg.last_profile is not None
+        assert not fg.trace.pending and not fg.trace.recording and fg.trace.last_path is not None
         traces_ = list(tmp_path.glob("fastgen_*.json.gz"))
-        assert len(traces_) == 1 and str(traces_[0]) == fg.last_profile
+        assert len(traces_) == 1 and str(traces_[0]) == fg.trace.last_path
         with gzip.open(traces_[0], "rt") as f:
             text = f.read()
         assert "traceEvents" in text and ("gemm_skinny" in text or "attn_" in text)  # the engine's kernels are in it

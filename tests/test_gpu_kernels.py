@@ -414,7 +414,7 @@ def test_gemm_skinny_gate_up_epilogue(ops, M, F, K):
     assert (got - want).abs().max() <= 1e-2 * want.abs().max() + 1e-3
 
 
-@pytest.mark.parametrize("M", [1, 2, 8, 16])
+@pytest.mark.parametrize("M", [1, 2, 8, 11, 16])
 @pytest.mark.parametrize("N,K,F", [(240, 328, 200), (4096, 14336, 1000), (104, 64, 24), (520, 240, 328)])
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
 def test_norms_folded_into_the_products(ops, M, N, K, F, w_dtype):
@@ -448,6 +448,13 @@ def test_norms_folded_into_the_products(ops, M, N, K, F, w_dtype):
         g, u = normed @ wg.float().T, normed @ wu.float().T
         want = g * torch.sigmoid(g) * u
         assert (act - want).abs().max() <= 1.5e-2 * want.abs().max() + 1e-3
+    # the same consumers through the wide kernel (64 columns a workgroup), which takes such rows too
+    y = ops.gemm_skinny(sr, w2.to(DEV), wide=True).cpu().float()
+    assert (y - normed @ w2.float().T).abs().max() <= 1.5e-2 * (normed @ w2.float().T).abs().max() + 1e-3
+    if F % 8 == 0:
+        act = ops.gemm_skinny(sr, ops.interleave_gate_up(wg, wu).contiguous().to(DEV), silu_mul_epilogue=True,
+                              wide=True).cpu().float()
+        assert (act - want).abs().max() <= 1.5e-2 * want.abs().max() + 1e-3
     h2 = torch.randn(M, F)
     h2_d = h2.to(DEV)
     nw2 = 1 + 0.1 * torch.randn(F)
@@ -455,6 +462,23 @@ def test_norms_folded_into_the_products(ops, M, N, K, F, w_dtype):
     want_h2 = h2 + normed @ w2.float().T
     assert torch.allclose(h2_d.cpu(), want_h2, atol=1.5e-2 * float(want_h2.abs().max()))
     assert sr2.ssq.shape == (M, -(-F // 16))
+
+
+@pytest.mark.parametrize("M", [1, 8, 9, 16, 17, 64, 200])
+def test_logits_product_at_a_whole_vocabulary(ops, M):
+    """``linear(x, w, out_dtype=float32)`` as the head calls it, at the size of a real vocabulary (128,256 rows
+    of 4,096): every kernel that takes it, by the number of rows, against a float64 product of the same bfloat16
+    operands."""
+    from fastgen_amd.kernels.linear import linear
+
+    torch.manual_seed(M)
+    N, K = 128256, 4096
+    x = torch.randn(M, K).bfloat16().to(DEV)
+    w = (torch.randn(N, K, device=DEV) * K**-0.5).bfloat16()
+    y = linear(x, w, out_dtype=torch.float32)
+    assert y.dtype == torch.float32 and y.shape == (M, N)
+    want = x.double() @ w.double().T
+    assert float((y.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
 
 
 @pytest.mark.parametrize("M", [1, 5, 16])

@@ -152,6 +152,38 @@ def test_llama3_frequencies():
         assert math.isclose(float(got), fr / expect_div, rel_tol=1e-4)
 
 
+@pytest.mark.parametrize("head_dim,theta,sc", [
+    (128, 500000.0, dict(factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)),
+    (128, 500000.0, dict(factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)),
+    (256, 10000.0, dict(factor=3.0, low_freq_factor=2.0, high_freq_factor=16.0, original_max_position_embeddings=96)),
+])
+def test_llama3_blend_is_affine_in_the_frequency(head_dim, theta, sc):
+    """What fixes the middle band beside the reference's text (fastgen/forward.py:630-633): the blend's
+    variable is ``ctx / wavelength = ctx * f / (2 pi)``, so ``f' / f = (1 - x) / factor + x`` is affine in the
+    frequency ``f``, with the values 1 / factor and 1 at the band's two edges.  An affine function with those
+    two values is one function: a blend that is linear in the wavelength (or in the index, or in log f) equals
+    it at the edges and nowhere between, and fails here."""
+    base = plain_rope_frequencies(head_dim, theta).double()
+    f = plain_rope_frequencies(head_dim, theta, sc).double()
+    ctx, lo_f, hi_f, factor = (sc["original_max_position_embeddings"], sc["low_freq_factor"], sc["high_freq_factor"],
+                               sc["factor"])
+    f_lo, f_hi = 2 * math.pi * lo_f / ctx, 2 * math.pi * hi_f / ctx  # frequencies of the band's edges
+    mid = (base > f_lo * 1.001) & (base < f_hi * 0.999)
+    assert int(mid.sum()) >= 3, "the test needs three frequencies inside the band"
+    ratio = f[mid] / base[mid]
+    # the affine function through (f_lo, 1 / factor) and (f_hi, 1)
+    want = 1 / factor + (base[mid] - f_lo) / (f_hi - f_lo) * (1 - 1 / factor)
+    assert torch.allclose(ratio, want, rtol=2e-5, atol=0), (ratio, want)
+    # equal slopes between neighbours (affine), and the plausible mistakes are far from it
+    slopes = (ratio[1:] - ratio[:-1]) / (base[mid][1:] - base[mid][:-1])
+    assert torch.allclose(slopes, slopes[0].expand_as(slopes), rtol=1e-3)
+    wl, wl_lo, wl_hi = 2 * math.pi / base[mid], ctx / lo_f, ctx / hi_f
+    in_wavelength = 1 / factor + (wl_lo - wl) / (wl_lo - wl_hi) * (1 - 1 / factor)
+    assert float((in_wavelength - want).abs().max()) > 0.05
+    in_log = 1 / factor + (base[mid].log() - math.log(f_lo)) / (math.log(f_hi) - math.log(f_lo)) * (1 - 1 / factor)
+    assert float((in_log - want).abs().max()) > 0.05
+
+
 # ---------------------------------------------------------------- attention
 @pytest.mark.parametrize("H,KV", [(4, 4), (4, 2), (6, 1), (1, 1)])
 def test_attention_is_the_library_routine(H, KV):

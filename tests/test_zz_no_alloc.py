@@ -15,27 +15,32 @@ from test_gpu_kernels import DEV, _paged_case, _plain_rows
 pytestmark = pytest.mark.gpu
 
 
-def _static_call(lib, case, items, n_items, max_chunks, min_tiles, max_rows, H, KV, hd, P, out):
+def _static_call(lib, case, items, n_items, max_chunks, min_tiles, max_rows, H, KV, hd, P, out, window=0):
     from fastgen_amd.kernels.ops import _ptr, _stream
 
     q = case["q"]
     return lib.fg_attn_decode_static(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(case["kp"]), _ptr(case["vp"]), _ptr(case["table"]),
         case["table"].stride(0), _ptr(items), n_items, max_chunks, min_tiles, max_rows, H, KV, hd, P,
-        ctypes.c_float(hd ** -0.5), 0, _stream(q))
+        ctypes.c_float(hd ** -0.5), window, _stream(q))
 
 
-@pytest.mark.parametrize("H,KV,hd,P", [(32, 8, 128, 64), (5, 1, 48, 32)])
-def test_decode_attention_without_allocation(H, KV, hd, P):
+@pytest.mark.parametrize("H,KV,hd,P,window,n_new", [(32, 8, 128, 64, 0, 1), (5, 1, 48, 32, 0, 1),
+                                                    (32, 8, 128, 64, 100, 1), (32, 8, 128, 64, 0, 2),
+                                                    (5, 1, 48, 32, 100, 2)])
+def test_decode_attention_without_allocation(H, KV, hd, P, window, n_new):
+    """``window``: keys further back than that are not seen (the plan then starts behind key 0);
+    ``n_new``: tokens an item brings (two tokens of a group of at most 8 heads are one item of at most 16 rows)."""
     from fastgen_amd.kernels import _lib, ops
 
     lib = _lib.load(f"attention_mfma@{hd}")
     lib.fg_attn_decode_static_error.restype = ctypes.c_char_p
     G = H // KV
+    assert G * n_new <= 16
     # the first call: many sequences, some long (several chunks each); the second: fewer and shorter
     calls = [
-        [(n, 1) for n in (700, 64, 1500, 3, 255, 256, 1023, 90, 2100, 17, 333, 640)],
-        [(n, 1) for n in (300, 5, 129)],
+        [(n, n_new) for n in (700, 64, 1500, 3, 255, 256, 1023, 90, 2100, 17, 333, 640)],
+        [(n, n_new) for n in (300, 5, 129)],
     ]
     n_calls = 0
     for min_tiles in (4, 1):
@@ -52,12 +57,12 @@ def test_decode_attention_without_allocation(H, KV, hd, P):
             # the existing entry points, with buffers that torch allocates
             want = torch.full_like(case["q"], float("nan"))
             ops.paged_attention_mfma(case["q"], want, case["kp"], case["vp"], case["table"], items, None, H,
-                                     hd ** -0.5, 0, None, max_chunks, min_tiles, max_rows=G)
+                                     hd ** -0.5, window, None, max_chunks, min_tiles, max_rows=G * n_new)
             got = torch.full_like(case["q"], float("nan"))
             torch.cuda.synchronize()
             before = torch.cuda.memory_stats()["allocation.all.allocated"]
             free_before = torch.cuda.mem_get_info()[0]
-            st = _static_call(lib, case, items, n, max_chunks, min_tiles, G, H, KV, hd, P, got)
+            st = _static_call(lib, case, items, n, max_chunks, min_tiles, G * n_new, H, KV, hd, P, got, window)
             assert st == 0, lib.fg_attn_decode_static_error().decode()
             assert torch.cuda.memory_stats()["allocation.all.allocated"] == before  # torch was asked for nothing
             torch.cuda.synchronize()
@@ -66,7 +71,7 @@ def test_decode_attention_without_allocation(H, KV, hd, P):
             n_calls += 1
             assert torch.isfinite(got).all()
             assert torch.equal(got, want)  # the same kernels with the same cut: the same bits
-            assert torch.allclose(got.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
+            assert torch.allclose(got.cpu().float(), _plain_rows(case, seqs, window or None), atol=1.5e-2, rtol=2e-2)
 
 
 def test_sizes_beyond_the_static_array_are_refused():
