@@ -42,6 +42,7 @@ LIBRARIES: Dict[str, str] = {
     "attention": "attention.hip",
     "gemm": "gemm.hip",
     "gemm_skinny": "gemm_skinny.hip",
+    "gemm_tiled": "gemm_tiled.hip",
     "sampling": "sampling.hip",
 }
 

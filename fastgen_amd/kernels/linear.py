@@ -43,6 +43,10 @@ def _library_mm_f32_out(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tens
 # what the kernels take (their limits, not a model's sizes)
 SKINNY_ROWS = 16  # one 16-row block of x: the narrow kernel (16 output columns a workgroup) and every folded epilogue
 WIDE_ROWS = ops.SKINNY_MAX_ROWS  # the wide kernel (64 columns a workgroup): up to eight blocks of x
+# the tiled kernel takes any number of rows; it is offered where it has been seen to win or come close (from the
+# wide kernel's range up to a few hundred rows; beyond, the library's large tiles are twice as fast)
+TILED_MIN_ROWS, TILED_MAX_ROWS = 65, 512
+TILED_TILES = ((0, 128), (2, 256))  # (config of ops.gemm_tiled, rows of its tile), both 128 columns wide
 
 
 def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -82,22 +86,34 @@ _TIMED_RUNS = 4
 
 def row_bucket(rows: int) -> int:
     """Products of up to 16 rows are measured per number of rows, above that per block of 16 rows
-    (the kernels work on such blocks), above the widest own kernel as one."""
+    (the kernels work on such blocks) up to 256, per block of 64 up to the last size at which an own
+    kernel is offered, and as one beyond."""
     if rows <= SKINNY_ROWS:
         return rows
-    return min(-(-rows // 16) * 16, WIDE_ROWS + 16)
+    if rows <= 256:
+        return -(-rows // 16) * 16
+    return min(-(-rows // 64) * 64, TILED_MAX_ROWS + 64)
+
+
+def tiled_splits(n_out: int, k: int, rows: int, tile_rows: int) -> int:
+    """Splits of the k range that give the tiled kernel about two workgroups a compute unit, at most 16,
+    each with at least 512 of k."""
+    tiles = -(-rows // tile_rows) * -(-n_out // 128)
+    return max(1, min(16, 2 * ops.compute_units() // tiles, k // 512))
 
 
 def _capturing() -> bool:
     return torch.cuda.is_current_stream_capturing()
 
 
-def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Callable[[], torch.Tensor]]]) -> str:
+def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Callable[[], torch.Tensor]]],
+            handicap: Optional[Dict[str, float]] = None) -> str:
     """The candidate to run: the forced one, the one the table holds, or the one that is fastest now.
     Timing needs the device to itself (events and a wait for them), so a product that is first met while
     a step is being recorded runs the first candidate, unrecorded in the table; the engine runs every
     step once, unrecorded, before it records it.  The candidates are timed in turn on the same
-    operands, each run behind a run of the other."""
+    operands, each run behind a run of the other.  ``handicap``: milliseconds added to a candidate's time
+    for what its result costs the consumer (partial sums that are still to be added)."""
     names = [c[0] for c in candidates]
     if force in names:
         return force
@@ -121,7 +137,7 @@ def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Ca
             ev[r][1].record()
     torch.cuda.current_stream().synchronize()
     for ev, name in zip(events, names):
-        best[name] = min(a.elapsed_time(b) for a, b in ev)
+        best[name] = min(a.elapsed_time(b) for a, b in ev) + (handicap or {}).get(name, 0.0)
     winner = min(names, key=lambda nm: best[nm])
     choices[key] = winner
     return winner
@@ -182,22 +198,38 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         return ops.silu_mul(y) if silu else y
 
     candidates: List[Tuple[str, Callable[[], torch.Tensor]]] = []
+    handicap: Dict[str, float] = {}
+    tiled_ok = own and TILED_MIN_ROWS <= rows <= TILED_MAX_ROWS
+
+    def sums_cost(splits: int) -> float:
+        """Milliseconds the consumer takes to read the partial sums beyond the first (at 4 TB/s)."""
+        return (splits - 1) * rows * N * 4 / 4e9
+
     if own and silu and out_dtype == torch.bfloat16 and N % 16 == 0:
         if rows <= SKINNY_ROWS:
             candidates.append(("narrow", lambda: ops.gemm_skinny(src, w, silu_mul_epilogue=True, wide=False)))
         if rows <= WIDE_ROWS:
             candidates.append(("wide", lambda: ops.gemm_skinny(src, w, silu_mul_epilogue=True, wide=True)))
+        if tiled_ok:
+            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, w, silu_mul_epilogue=True, config=TILED_TILES[1][0])))
     elif own and not silu:
         if rows <= SKINNY_ROWS:
             candidates.append(("narrow", lambda: ops.gemm_skinny(src, w, out_dtype, wide=False)))
         elif rows <= WIDE_ROWS and partials_ok:
             splits = k_splits_for(N, K, rows)
             candidates.append(("wide", lambda: ops.gemm_skinny(x, w, out_dtype, k_splits=splits, wide=True)))
+            handicap["wide"] = sums_cost(splits)
         elif rows <= 64:
             candidates.append(("wide", lambda: ops.gemm_skinny(x, w, out_dtype, wide=True)))
+        if tiled_ok and partials_ok and out_dtype == torch.bfloat16:
+            for name, (config, tile_rows) in zip(("tiled", "tiled256"), TILED_TILES):
+                s_t = tiled_splits(N, K, rows, tile_rows)
+                candidates.append((name, lambda config=config, s_t=s_t: ops.gemm_tiled(x, w, out_dtype, k_splits=s_t,
+                                                                                       config=config)))
+                handicap[name] = sums_cost(s_t)
     if scaled is None or not candidates:
         candidates.append(("library", library))
     what = ("silu_mul" if silu else "store") + ("+partials" if partials_ok and rows > SKINNY_ROWS else "") + (
         "+f32" if out_dtype == torch.float32 else "") + ("+scaled" if scaled is not None else "")
-    name = _choose(what, N, K, rows, candidates)
+    name = _choose(what, N, K, rows, candidates, handicap)
     return dict(candidates)[name]()

@@ -215,6 +215,25 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, sil
     return y.to(out_dtype or torch.bfloat16)
 
 
+def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+               silu_mul_epilogue: bool = False, k_splits: int = 1, config: int = 0) -> torch.Tensor:
+    """``x @ w.T``; with ``silu_mul_epilogue`` as :func:`gemm_skinny`; with ``k_splits > 1`` fp32 ``[S, M, N]``
+    partial sums over the k ranges ``[s * ceil(K / S / 32) * 32, ...)``.  ``config`` only picks a tile."""
+    xf, wf = x.float(), w.float()
+    if k_splits > 1:
+        K = wf.shape[1]
+        step = -(-K // (k_splits * 32)) * 32
+        return torch.stack([xf[:, s * step : (s + 1) * step] @ wf[:, s * step : (s + 1) * step].T
+                            for s in range(k_splits)])
+    y = xf @ wf.T
+    if silu_mul_epilogue:
+        M, N = y.shape
+        gu = y.view(M, N // 16, 2, 8)
+        g, u = gu[:, :, 0].reshape(M, N // 2), gu[:, :, 1].reshape(M, N // 2)
+        y = g * torch.sigmoid(g) * u
+    return y.to(out_dtype or torch.bfloat16)
+
+
 def gemm_skinny_residual(x, w: torch.Tensor, h: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
     """``h += x @ w.T``; returns what the RMSNorm after it needs: ``h * norm_weight`` in bfloat16 and the sums of
     squares of ``h`` over each block of 16 columns."""

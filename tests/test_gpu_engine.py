@@ -282,12 +282,13 @@ def test_many_requests_decode_together_bfloat16(n_live, captured, tmp_path):
                  plain_logits(weights, cfg, tokens, torch.bfloat16), f"{n_live} live")
 
 
-@pytest.mark.parametrize("forced", ["narrow", "wide", "library", None])
+@pytest.mark.parametrize("forced", ["narrow", "wide", "tiled", "tiled256", "library", None])
 def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, tmp_path, monkeypatch):
     """Which kernel takes a matrix product is measured at run time (``fastgen_amd.kernels.linear``), so which
     one an engine test meets depends on the machine.  Here the engine runs once under each kernel's name
-    (taken wherever it is among the candidates of a product) and once as measured: mixed steps, and 20
-    requests decoding together (17..32 rows), every position against the plain implementation."""
+    (taken wherever it is among the candidates of a product) and once as measured: whole prompts (up to 150
+    rows), mixed steps, and 20 requests decoding together (17..32 rows), every position against the plain
+    implementation."""
     from fastgen_amd.kernels import linear
 
     monkeypatch.setattr(linear, "force", forced)
@@ -299,11 +300,11 @@ def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, tmp_path
     lengths = {"a": 100, "b": 33, "c": 64, "d": 7, "e": 150}
     g = torch.Generator().manual_seed(13)
     tokens = {rid: torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for rid, n in lengths.items()}
-    trace = traces.mixed(lengths, seed=3)
-    runner = make_runner(folder, torch.bfloat16, 32, traces.max_live_tokens(trace, 64))
-    got = run_trace(runner, trace, tokens)
-    assert_close(got, plain_logits(weights, cfg, tokens), torch.bfloat16,
-                 plain_logits(weights, cfg, tokens, torch.bfloat16), f"forced {forced}, mixed")
+    want, noise = plain_logits(weights, cfg, tokens), plain_logits(weights, cfg, tokens, torch.bfloat16)
+    for name, trace in (("whole", traces.whole(lengths)), ("mixed", traces.mixed(lengths, seed=3))):
+        runner = make_runner(folder, torch.bfloat16, 32, traces.max_live_tokens(trace, 64))
+        got = run_trace(runner, trace, tokens)
+        assert_close(got, want, torch.bfloat16, noise, f"forced {forced}, {name}")
     prompts = {f"r{i}": 5 + 3 * i for i in range(20)}
     tokens = {rid: torch.randint(0, cfg["vocab_size"], (n + 12,), generator=g).tolist() for rid, n in prompts.items()}
     trace = traces.many_decoding_together(prompts, 12, seed=1)
@@ -312,4 +313,4 @@ def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, tmp_path
     assert_close(got, plain_logits(weights, cfg, tokens), torch.bfloat16,
                  plain_logits(weights, cfg, tokens, torch.bfloat16), f"forced {forced}, 20 live")
     if forced is None:
-        assert linear.choices and set(linear.choices.values()) <= {"narrow", "wide", "library"}
+        assert linear.choices and set(linear.choices.values()) <= {"narrow", "wide", "tiled", "tiled256", "library"}

@@ -23,7 +23,7 @@ from plain_llama import plain_attention, plain_rmsnorm, plain_rope_interleaved, 
 # functions of ops that launch a kernel (the others plan work, build arguments or pick a kernel)
 KERNEL_OPS = ["embed", "add_rmsnorm", "rmsnorm", "silu_mul", "rope_table", "rope_kv_write", "paged_attention_general",
               "paged_attention_mfma", "paged_attention", "gemm_nt", "scale_rows", "gemm_skinny_residual", "gemm_skinny",
-              "gemm_skinny_qkv", "sample", "logprob"]
+              "gemm_skinny_qkv", "gemm_tiled", "sample", "logprob"]
 
 
 @pytest.mark.parametrize("name", KERNEL_OPS + ["interleave_gate_up"])
@@ -306,6 +306,20 @@ def test_gemm_skinny_twins(ops, M, N, K):
             _close(ops.gemm_skinny(folded_g, w2.cuda(), wide=wide), twins.gemm_skinny(folded_c, w2, wide=wide), bf)
             _close(ops.gemm_skinny(folded_g, w2.cuda(), None, True, 1, wide),
                    twins.gemm_skinny(folded_c, w2, None, True, 1, wide), bf)
+
+
+@gpu
+@pytest.mark.parametrize("M,N,K", [(130, 48, 72), (300, 528, 1032), (70, 272, 520)])
+def test_gemm_tiled_twins(ops, M, N, K):
+    torch.manual_seed(N)
+    bf = torch.bfloat16
+    x, w = (torch.randn(M, K) / 4).to(bf), (torch.randn(N, K) / 4).to(bf)
+    for config in range(kernel_ops.TILED_CONFIGS):
+        _both("gemm_tiled", lambda: (x, w, None, False, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, torch.float32, False, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, None, True, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, None, False, 3, config),
+              lambda g, t, *_: (_close(g.sum(0), t.sum(0), bf), torch.testing.assert_close(g.cpu(), t, rtol=2e-3, atol=2e-3)), ops)
 
 
 @gpu
