@@ -57,6 +57,24 @@ SHAPES = {"3b": ("llama-3.2-3b-shape-random", LLAMA_3B), "8b": ("llama-3.1-8b-sh
           "70b": ("llama-3.1-70b-shape-random", LLAMA_70B)}
 
 
+def workload_roofline(engine, cfg: dict, seconds: float) -> dict:
+    """Where a whole run stands against the two rooflines: the bytes its steps had to read (every weight once
+    a step, and the cache of every request in the step) over the time and the HBM peak; the flops of its matrix
+    products and attention over the time and the bf16 MFMA peak.  A run is bound by neither alone (its prompt
+    steps by the matrix cores, its decode steps by memory), so the two fractions together say how much of the
+    GPU it used."""
+    D, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    H, KV, L = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["num_hidden_layers"]
+    hd = D // H
+    layer_params = D * (H + 2 * KV) * hd + H * hd * D + 3 * D * F
+    w = engine.work
+    weight_bytes = (L * layer_params + D * V) * 2
+    nbytes = w.steps * weight_bytes + w.cache_reads * 2 * KV * hd * 2 * L
+    flops = 2 * w.tokens * L * layer_params + 4 * H * hd * L * w.keys_attended
+    return {"hbm_frac": round(nbytes / seconds / PEAK_HBM, 4), "mfma_frac": round(flops / seconds / PEAK_FLOPS["bf16"], 4),
+            "gbytes": round(nbytes / 1e9, 1), "tflop": round(flops / 1e12, 1), "steps": w.steps, "tokens": w.tokens}
+
+
 def serve_workload(n_requests: int = 256, step_budget: int = 2048, shape: str = "3b") -> int:
     """Continuous batching at the Llama 3.2 3B shape (random bfloat16 weights): ``n_requests`` requests
     arrive at once, prompts of 128..4096 uniform random ids, 32..512 greedy tokens each, at most 256 live,
@@ -93,6 +111,7 @@ def serve_workload(n_requests: int = 256, step_budget: int = 2048, shape: str = 
     print(json.dumps({
         "metric": "generated tok/s, continuous batching", "value": round(sum(olens) / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "roofline": workload_roofline(engine, cfg, dt),
         "config": {"model": model_name, "requests": n_requests, "prompt_tokens": sum(plens),
                    "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": step_budget, "page_size": PAGE,
                    "engine_steps": engine.n_steps, "preemptions": engine.scheduler.n_preemptions},
@@ -150,6 +169,7 @@ def readme_workload(shape: str = "8b") -> int:
         "metric": "generated tok/s, 512 prompts x 1024 tokens, 128 decode steps", "value": round(generated / dt, 1),
         "unit": "tokens/s", "n_gpus": 1, "seconds": round(dt, 3), "higher_is_better": True, "dtype": "bf16",
         "data": "synthetic", "vs_published": round(generated / dt / published[0], 3) if published else None,
+        "roofline": workload_roofline(engine, cfg, dt),
         "config": {"model": model_name, "requests": n, "prompt_len": p_len, "generated": n_gen,
                    "max_batch": max_batch, "step_budget": 8192, "page_size": PAGE, "engine_steps": engine.n_steps,
                    "cache_tokens": pool, "cache": "free memory after the weights",

@@ -776,17 +776,20 @@ extern "C" int fg_attn_decode_static(const void* q, int q_stride, void* out, int
 // compute unit holds one workgroup whose eight waves all work until its end.  Workgroups are
 // launched in the order of the items (most keys first), so short ones fill in behind long ones.
 // Above 128: 4 waves of 16 rows, one tile at a time (two tiles would not fit the 64 KB of LDS).
-constexpr bool TILE_PAIR = HD <= 128;
-constexpr int TILE_RB = TILE_PAIR ? 2 : 1;         // row blocks a wave holds
-constexpr int TILE_ROWS = 64 * TILE_RB;            // query rows of an item
-constexpr int TILE_THREADS = TILE_PAIR ? 512 : 256;
+// The second form also serves head sizes up to 128 when a step has few items ("small" items of 64 rows:
+// twice as many workgroups of half the size, several to a compute unit, out of step with one another).
+constexpr bool TILE_PAIR_OK = HD <= 128;
+constexpr int TILE_ROWS = TILE_PAIR_OK ? 128 : 64;   // query rows of an item of the first form that this head size has
+constexpr int TILE_ROWS_SMALL = 64;                // of the second form
 
-template <bool PERM>
-__global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
+template <bool PERM, bool TILE_PAIR>
+__global__ __launch_bounds__(TILE_PAIR ? 512 : 256, TILE_PAIR ? 1 : 2) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ items, int n_heads, int n_kv,
     int page_size, int page_shift, float scale, int window) {
+  constexpr int TILE_RB = TILE_PAIR ? 2 : 1;  // row blocks a wave holds
+  constexpr int TILE_THREADS = TILE_PAIR ? 512 : 256;
   constexpr int NT = TILE_THREADS;
   constexpr int NPT = TILE_PAIR ? 2 : 1;    // tiles a pass of the loop takes
   // tiles in LDS: with pairs, one pair is read while the next is written (128 KB at head size 128, of
@@ -1055,22 +1058,43 @@ __global__ __launch_bounds__(TILE_THREADS, 1) void attn_tile_kernel(
   }
 }
 
+struct TileArgs {
+  const bf16_t* q; int q_stride; bf16_t* out; int out_stride; const bf16_t* k_pages; const bf16_t* v_pages;
+  const int* block_table; int bt_stride; const int* items; int n_items, n_heads, n_kv, page_size; float scale;
+  int window; hipStream_t stream;
+};
+template <bool PERM, bool PAIR>
+static void launch_tile(const TileArgs& a) {
+  attn_tile_kernel<PERM, PAIR><<<a.n_items * a.n_kv, PAIR ? 512 : 256, 0, a.stream>>>(
+      a.q, a.q_stride, a.out, a.out_stride, a.k_pages, a.v_pages, a.block_table, a.bt_stride, a.items, a.n_heads,
+      a.n_kv, a.page_size, page_shift_of(a.page_size), a.scale, a.window);
+}
+// the form with two tiles at a time exists up to head size 128 only (its LDS)
+template <bool EXISTS> struct PairForm {
+  static void go(const TileArgs& a) {
+    if (a.page_size % 32 == 0) launch_tile<true, true>(a); else launch_tile<false, true>(a);
+  }
+};
+template <> struct PairForm<false> { static void go(const TileArgs&) {} };
+
+// item_rows: the rows an item has at most, fg_attn_tile_rows(0) or fg_attn_tile_rows(1): which form of the kernel runs.
 extern "C" int fg_attn_tile(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                             const void* v_pages, const int* block_table, int bt_stride, const int* items,
-                            int n_items, int n_heads, int n_kv, int hd, int page_size, float scale, int window,
-                            hipStream_t stream) {
+                            int n_items, int item_rows, int n_heads, int n_kv, int hd, int page_size, float scale,
+                            int window, hipStream_t stream) {
   if (n_items <= 0) return FG_OK;
-  if (hd != HD || !(scale > 0.f) || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > TILE_ROWS || page_size < 8 || page_size % 8 ||
-      (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4)
+  if (hd != HD || !(scale > 0.f) || n_kv <= 0 || n_heads % n_kv || n_heads / n_kv > item_rows || page_size < 8 || page_size % 8 ||
+      (long long)n_items * n_kv > 2147483647LL || window < 0 || q_stride % 8 || out_stride % 4 ||
+      (item_rows != TILE_ROWS && item_rows != TILE_ROWS_SMALL))
     return FG_ERR_ARG;
-#define LAUNCH(PERM)                                                                                        \
-  attn_tile_kernel<PERM><<<n_items * n_kv, TILE_THREADS, 0, stream>>>(                                      \
-      (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
-      block_table, bt_stride, items, n_heads, n_kv, page_size, page_shift_of(page_size), scale, window)
-  if (page_size % 32 == 0) LAUNCH(true); else LAUNCH(false);
-#undef LAUNCH
+  const TileArgs a{(const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,
+                   block_table, bt_stride, items, n_items, n_heads, n_kv, page_size, scale, window, stream};
+  if (TILE_PAIR_OK && item_rows == TILE_ROWS) PairForm<TILE_PAIR_OK>::go(a);
+  else if (page_size % 32 == 0) launch_tile<true, false>(a);
+  else launch_tile<false, false>(a);
   return fg_launch_status();
 }
 
-// query rows (tokens x heads of a kv head's group) of one item of fg_attn_tile
-extern "C" int fg_attn_tile_rows() { return TILE_ROWS; }
+// query rows (tokens x heads of a kv head's group) of one item of fg_attn_tile: of the larger form, or
+// (small != 0) of the form with 64-row items
+extern "C" int fg_attn_tile_rows(int small) { return small ? TILE_ROWS_SMALL : TILE_ROWS; }

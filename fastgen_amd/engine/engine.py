@@ -52,6 +52,25 @@ def step_memory_estimate(model: Model, max_step_tokens: int, max_batch: int) -> 
     return int(max_step_tokens * 12 * widest + 3 * max_batch * model.vocab_size * 4)
 
 
+@dataclass
+class WorkDone:
+    """What the engine's steps have asked of the GPU so far, for measurements: ``steps`` runs of the model
+    (each reads every weight once), ``tokens`` run through it, ``cache_reads``: over all steps and their
+    requests, the cached tokens of the request after the step (what its attention reads at least once),
+    ``keys_attended``: over all tokens, the keys each attends (its attention's products)."""
+
+    steps: int = 0
+    tokens: int = 0
+    cache_reads: int = 0
+    keys_attended: int = 0
+
+    def note(self, start: int, n: int) -> None:
+        """A request brought ``n`` tokens at positions ``start ..`` to one step."""
+        self.tokens += n
+        self.cache_reads += start + n
+        self.keys_attended += n * start + n * (n + 1) // 2
+
+
 class Engine:
     def __init__(self, model: Model, page_size: int = 64, max_tokens: Optional[int] = 8192, max_batch: int = 64,
                  max_step_tokens: int = 2048, max_seq: Optional[int] = None, seed: int = 0,
@@ -92,6 +111,7 @@ class Engine:
         self._held: List[Request] = []  # ended, with samples still on the device
         self._n_requests = 0
         self._logged_running = -1  # the batch size that the log line of the last decode run named
+        self.work = WorkDone()
         self.n_steps = 0
         self.last_mean_context = 0.0  # set by time_decode
 
@@ -170,6 +190,9 @@ class Engine:
                         len(sched.running), len(sched.waiting), n_tokens, n_tokens - len(rows))
         logits = self.runner.step(entries, prev.tokens if prev is not None else None)
         self.n_steps += 1
+        self.work.steps += 1
+        for e in plan:
+            self.work.note(e.start, e.n)
         tok = lps = None
         if rows:
             tok = self.sampler.sample(
@@ -236,6 +259,11 @@ class Engine:
         """``n_steps`` decode steps of all running requests with one look at the
         tokens at the end."""
         reqs = list(self.scheduler.running)
+        self.work.steps += n_steps
+        for r in reqs:
+            at = self.runner.cache.length(r.rid)  # the position of the token it brings to the first step
+            for s_ in range(n_steps):
+                self.work.note(at + s_, 1)
         entries = [StepEntry(r.rid, [r.generated[-1] if r.generated else r.prompt[-1]], [0]) for r in reqs]
         sample = self.sampler.prepare([r.temperature for r in reqs], [r.top_p for r in reqs],
                                       [r.seed for r in reqs], [len(r.generated) for r in reqs], n_steps)

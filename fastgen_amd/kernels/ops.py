@@ -292,9 +292,10 @@ def _split_target_blocks() -> int:
 _SPLIT_MIN_TILES = int(os.environ.get("FG_SPLIT_MIN_TILES", 4))
 
 
-def attention_tile_rows(head_dim: int) -> int:
-    """Query rows of one item of the tile kernel for this head size."""
-    return int(_lib.load(f"attention_mfma@{head_dim}").fg_attn_tile_rows())
+def attention_tile_rows(head_dim: int, small: bool = False) -> int:
+    """Query rows of one item of the tile kernel for this head size: of its larger form (128 rows up to
+    head size 128), or of the form with ``small`` items (64 rows, more and lighter workgroups)."""
+    return int(_lib.load(f"attention_mfma@{head_dim}").fg_attn_tile_rows(int(small)))
 
 
 def attention_items(q_lens, q_start, n_cached, group_size: int, tile_rows: int = 64):
@@ -352,13 +353,14 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
                          plan: Optional[torch.Tensor] = None, max_chunks: Optional[int] = None,
-                         min_tiles: int = 4, max_rows: int = 16) -> torch.Tensor:
+                         min_tiles: int = 4, max_rows: int = 16, tile_rows: Optional[int] = None) -> torch.Tensor:
     """bf16 attention on the matrix cores.  ``small_items`` / ``big_items`` are
     device int32 ``[n, 4]`` lists from :func:`attention_items` (16-byte aligned);
     every query token of the step must be covered by exactly one item.
     ``plan``: :func:`attention_plan` of the small items with this ``max_chunks``
     and ``window`` (made here if not given).  ``max_rows``: no small item has
-    more rows (tokens times query heads per kv head) than this."""
+    more rows (tokens times query heads per kv head) than this.  ``tile_rows``: the
+    rows the big items were cut for (:func:`attention_tile_rows`; default: the larger form's)."""
     _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
@@ -396,12 +398,14 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
             page_size, ctypes.c_float(scale), int(window or 0), _stream(q))
         _check(st, "attn_split")
     if big_items is not None and big_items.numel():
-        _need(G <= attention_tile_rows(hd), "too many query heads per kv head for the tile kernel")
+        tile_rows = attention_tile_rows(hd) if tile_rows is None else int(tile_rows)
+        _need(tile_rows in (attention_tile_rows(hd), attention_tile_rows(hd, True)), "tile_rows is no form of the tile kernel")
+        _need(G <= tile_rows, "too many query heads per kv head for the tile kernel")
         _i32(big_items, "big_items")
         _need(big_items.data_ptr() % 16 == 0, "items must be 16-byte aligned")
         st = lib.fg_attn_tile(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-            block_table.stride(0), _ptr(big_items), big_items.numel() // 4, n_heads, n_kv, hd, page_size,
+            block_table.stride(0), _ptr(big_items), big_items.numel() // 4, tile_rows, n_heads, n_kv, hd, page_size,
             ctypes.c_float(scale), int(window or 0), _stream(q))
         _check(st, "attn_tile")
     return out
@@ -422,18 +426,27 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
     if q.dtype != torch.bfloat16 or hd % 16 or hd > MFMA_MAX_HEAD_DIM or G > 16:
         return paged_attention_general(q, out, k_pages, v_pages, group.block_table, ctx.seq_of_token,
                                        ctx.positions, n_heads, scale, window)
-    plan = ctx.scratch.get(("attention_items", G))
+    items_key = ("attention_items", G, hd, n_kv)  # (how a step is cut into items depends on all three)
+    plan = ctx.scratch.get(items_key)
     if plan is None:
         if ctx.seq_records is not None and int(ctx.q_lens.max()) * G <= 16:
             # every sequence is one item of the split kernel: its records are in the step's buffer
             # already (and are refreshed with it when the step is a replayed graph)
-            plan = (ctx.seq_records, None, ctx.n_seqs)
+            plan = (ctx.seq_records, None, ctx.n_seqs, None)
         else:
-            small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, attention_tile_rows(hd))
+            tile_rows = attention_tile_rows(hd)
+            small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, tile_rows)
+            if 0 < len(big) * n_kv <= compute_units() // 2 and attention_tile_rows(hd, True) < tile_rows:
+                # so few items that half the compute units would stand idle: items of half the rows, whose
+                # lighter workgroups share a unit (prompt portions of up to 512 tokens: 11.6 / 17.6 us
+                # against 14.1 / 19.5 at 256 / 512 tokens; equal at 1,024, slower beyond)
+                tile_rows = attention_tile_rows(hd, True)
+                small, big = attention_items(ctx.q_lens, ctx.q_start_host, ctx.n_cached, G, tile_rows)
             both = upload(np.concatenate([small, big]).reshape(-1), torch.int32, q.device)
-            plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small))
-        ctx.scratch[("attention_items", G)] = plan
-    small_d, big_d, n_small = plan
+            plan = (both[: small.size] if small.size else None, both[small.size:] if big.size else None, len(small),
+                    tile_rows)
+        ctx.scratch[items_key] = plan
+    small_d, big_d, n_small, tile_rows = plan
     chunks = split_plan = None
     if n_small:
         # how the items' key ranges are cut depends on the window: layers with the same one share the cut
@@ -445,7 +458,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v
     # rows of the largest small item: one token a sequence in a decode step (also a captured one)
     rows = G * int(ctx.q_lens.max()) if big_d is None else 16
     return paged_attention_mfma(q, out, k_pages, v_pages, group.block_table, small_d, big_d, n_heads, scale,
-                                window, split_plan, chunks, max_rows=min(16, rows))
+                                window, split_plan, chunks, max_rows=min(16, rows), tile_rows=tile_rows)
 
 
 # ----------------------------------------------------------------------- gemm

@@ -151,7 +151,8 @@ def paged_attention_general(q: torch.Tensor, out: torch.Tensor, k_pages: torch.T
 def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
-                         plan=None, max_chunks=None, min_tiles: int = 4, max_rows: int = 16) -> torch.Tensor:
+                         plan=None, max_chunks=None, min_tiles: int = 4, max_rows: int = 16,
+                         tile_rows=None) -> torch.Tensor:
     """The same attention for tokens listed as items (sequence, first flat token, tokens, position of the
     first token).  How the kernels cut the work (``plan`` and what follows it) does not change the result."""
     seq_of_token = torch.zeros(q.shape[0], dtype=torch.int32)

@@ -660,20 +660,20 @@ def test_kernels_refuse_what_they_cannot_take(ops):
 CUTS = {"auto": (None, 4), "coarse": ("least", 4), "fine": (4096, 1), "pairs": (4096, 2)}
 
 
-def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto", max_rows=16):
+def _run_mfma(ops, case, seqs, H, KV, window=0, cut="auto", max_rows=16, small_tiles=False):
     import numpy as np
 
     q_lens = [b for _, b in seqs]
     q_start = np.concatenate([[0], np.cumsum(q_lens)])
-    small, big = ops.attention_items(q_lens, q_start, [a for a, _ in seqs], H // KV,
-                                     ops.attention_tile_rows(case["kp"].shape[3]))
+    tile_rows = ops.attention_tile_rows(case["kp"].shape[3], small_tiles)
+    small, big = ops.attention_items(q_lens, q_start, [a for a, _ in seqs], H // KV, tile_rows)
     dev = lambda a: torch.from_numpy(a.reshape(-1)).to(DEV) if a.size else None
     out = torch.full_like(case["q"], float("nan"))
     max_chunks, min_tiles = CUTS[cut]
     if max_chunks == "least":
         max_chunks = 2 * len(small)
     ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], dev(small), dev(big), H,
-                             case["kp"].shape[3] ** -0.5, window, None, max_chunks, min_tiles, max_rows)
+                             case["kp"].shape[3] ** -0.5, window, None, max_chunks, min_tiles, max_rows, tile_rows)
     return out, len(small), len(big)
 
 
@@ -693,10 +693,14 @@ MFMA_SEQS = [(0, 1), (0, 70), (131, 1), (60, 9), (17, 2), (255, 1), (0, 129), (3
 
 @pytest.mark.parametrize("H,KV,hd,P", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 37, 150])
-@pytest.mark.parametrize("cut", ["coarse", "fine"])
+@pytest.mark.parametrize("cut", ["coarse", "fine", "small tiles"])
 def test_paged_attention_mfma(ops, H, KV, hd, P, window, cut):
+    """``small tiles``: the prompt portions as items of 64 rows (the tile kernel's lighter form, which head sizes
+    above 128 always take) instead of 128."""
     case = _paged_case(torch.bfloat16, MFMA_SEQS, H, KV, hd, P, seed=21)
-    out, n_small, n_big = _run_mfma(ops, case, MFMA_SEQS, H, KV, window, cut)
+    small_tiles = cut == "small tiles"
+    out, n_small, n_big = _run_mfma(ops, case, MFMA_SEQS, H, KV, window, "coarse" if small_tiles else cut,
+                                    small_tiles=small_tiles)
     assert n_small and n_big  # both kernels run
     want = _plain_rows(case, MFMA_SEQS, window or None)
     assert torch.isfinite(out).all()  # every row written, no poison read
