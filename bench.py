@@ -200,6 +200,8 @@ def main() -> int:
                     help="decode (default): the step benchmark; serve: continuous batching of 256 requests; "
                          "readme: the load of the reference's README")
     ap.add_argument("--step-budget", type=int, default=2048, help="tokens a step of the serve workload")
+    ap.add_argument("--show-choices", action="store_true",
+                    help="print (stderr) which kernel the run's measurements chose for each matrix product")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported", flush=True)
@@ -292,6 +294,12 @@ def main() -> int:
         "points": {f"decode_b{b}": round(v["tok_s"], 1) for b, v in results.items() if b != a.batch},
     }
     print(json.dumps(line), flush=True)
+    if a.show_choices:
+        from fastgen_amd.kernels import linear
+
+        for (what, n, k, rows), name in sorted(linear.choices.items(), key=lambda kv: (kv[0][1], kv[0][2], kv[0][0], kv[0][3])):
+            took = ", ".join(f"{c} {1e3 * t:.1f} us" for c, t in sorted(linear.timings.get((what, n, k, rows), {}).items()))
+            print(f"[bench] product {what} N={n} K={k} rows<={rows}: {name} ({took})", file=sys.stderr)
     return 0
 
 

@@ -9,7 +9,7 @@ all of them: cuBLAS through ``F.linear``, ``fastgen/forward.py:433-513``).
 Which one is the fastest depends on the matrix and on the number of rows, so
 it is measured: the first time a product of some shape ``(N, K)`` meets some
 number of rows, the kernels that can take it are timed on the operands at hand
-and the winner is kept in one table (``choices``) for every later product of
+(the caches emptied before each run) and the winner is kept in one table (``choices``) for every later product of
 that shape and row bucket.  No size of any model stands here or in the parts.
 """
 
@@ -78,10 +78,18 @@ def k_splits_for(n_out: int, k: int, rows: int = 0) -> int:
 # ------------------------------------------------------------------ the table
 # (what is asked for, N, K, row bucket) -> name of the kernel that measured fastest
 choices: Dict[Tuple[str, int, int, int], str] = {}
+# the same keys -> what each candidate took when it was measured (milliseconds, the consumer's cost included)
+timings: Dict[Tuple[str, int, int, int], Dict[str, float]] = {}
 # set to a candidate's name to take that kernel wherever it is among the candidates (tests run the
 # engine once under each name, so that every kernel that may be chosen is compared with the plain run)
 force: Optional[str] = None
 _TIMED_RUNS = 4
+# Before each timed run this many bytes are read, so that a candidate finds the weights where a model's step
+# finds them: in memory, not in the caches (a memory-side cache of 256 MB and the L2s; a decode step streams
+# gigabytes of other weights between two uses of a matrix).  Timed warm, the wide kernel looks faster than the
+# narrow one on matrices that fit the cache and is the slower one in the model.  (Read, not written: modified
+# lines would be written back while the candidate runs, which costs the candidates unequally.)
+_FLUSH_BYTES = 384 << 20
 
 
 def row_bucket(rows: int) -> int:
@@ -112,7 +120,7 @@ def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Ca
     Timing needs the device to itself (events and a wait for them), so a product that is first met while
     a step is being recorded runs the first candidate, unrecorded in the table; the engine runs every
     step once, unrecorded, before it records it.  The candidates are timed in turn on the same
-    operands, each run behind a run of the other.  ``handicap``: milliseconds added to a candidate's time
+    operands, each run behind a sweep of memory that empties the caches.  ``handicap``: milliseconds added to a candidate's time
     for what its result costs the consumer (partial sums that are still to be added)."""
     names = [c[0] for c in candidates]
     if force in names:
@@ -128,18 +136,27 @@ def _choose(what: str, n: int, k: int, rows: int, candidates: List[Tuple[str, Ca
     best: Dict[str, float] = {}
     for fn in (c[1] for c in candidates):  # once each, unmeasured: libraries load, the library picks its kernel
         fn()
+    try:
+        flush = torch.zeros(_FLUSH_BYTES // 4, dtype=torch.int32, device=torch.cuda.current_device())
+        torch.cuda.current_stream().synchronize()  # (its zeros are in memory before anything is timed)
+    except RuntimeError:  # no memory to spare: the candidates are timed on what the caches hold
+        flush = None
     events = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
                for _ in range(_TIMED_RUNS)] for _ in candidates]
     for r in range(_TIMED_RUNS):
         for ev, (_, fn) in zip(events, candidates):
+            if flush is not None:
+                flush.amax()
             ev[r][0].record()
             fn()
             ev[r][1].record()
     torch.cuda.current_stream().synchronize()
+    del flush
     for ev, name in zip(events, names):
         best[name] = min(a.elapsed_time(b) for a, b in ev) + (handicap or {}).get(name, 0.0)
     winner = min(names, key=lambda nm: best[nm])
     choices[key] = winner
+    timings[key] = best
     return winner
 
 
