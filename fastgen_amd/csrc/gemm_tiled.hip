@@ -178,16 +178,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(
   }
 }
 
-// Tile shapes: waves as rows x columns of 64 x 64 each, stages of the ring.
-//   0: 2 x 2 waves (128 rows x 128 columns), 4 stages (64 KB: two workgroups a compute unit)
-//   1: 2 x 2 waves, 8 stages (128 KB)
-//   2: 4 x 2 waves (256 rows x 128 columns), 4 stages (96 KB)
-//   3: 2 x 4 waves (128 rows x 256 columns), 4 stages (96 KB)
-//   4: 4 x 2 waves, 6 stages (144 KB)
-#define FG_TILED_CONFIGS 5
-extern "C" int fg_gemm_tiled_rows(int config) { return config == 2 || config == 4 ? 256 : 128; }
-extern "C" int fg_gemm_tiled_cols(int config) { return config == 3 ? 256 : 128; }
-
+// Tile shapes (waves as rows x columns of 64 x 64 each), both with a ring of 4 stages:
+//   tile_rows 128: 2 x 2 waves, 128 rows x 128 columns (64 KB of LDS: two workgroups a compute unit)
+//   tile_rows 256: 4 x 2 waves, 256 rows x 128 columns (96 KB)
+// (Measured and dropped: rings of 6 and 8 stages, and 128 rows x 256 columns: never faster than these two.)
 template <int WM, int WN, int NST, int EPI, class TY>
 static int launch_tiled(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, long long part_stride,
                         int k_splits, int M, int N, int K, int k_per_split, hipStream_t stream) {
@@ -211,11 +205,11 @@ static int launch_tiled(const void* x, int ldx, const void* w, int ldw, void* y,
 // epilogue 1: w's rows are gate/up interleaved in groups of 8 (N % 16 == 0), y [M, N / 2] bf16 =
 // silu(gate) * up; k_splits must be 1.
 extern "C" int fg_gemm_tiled(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, long long part_stride,
-                             int k_splits, int M, int N, int K, int out_dtype, int epilogue, int config,
+                             int k_splits, int M, int N, int K, int out_dtype, int epilogue, int tile_rows,
                              hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
   if (K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535 ||
-      config < 0 || config >= FG_TILED_CONFIGS)
+      (tile_rows != 128 && tile_rows != 256))
     return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
@@ -231,13 +225,8 @@ extern "C" int fg_gemm_tiled(const void* x, int ldx, const void* w, int ldw, voi
     else if (out_dtype == FG_BF16) GO(WM, WN, NST, EPI_STORE, bf16_t);      \
     else GO(WM, WN, NST, EPI_STORE, float);                                 \
   } while (0)
-  switch (config) {
-    case 0: PICK(2, 2, 4);
-    case 1: PICK(2, 2, 8);
-    case 2: PICK(4, 2, 4);
-    case 3: PICK(2, 4, 4);
-    default: PICK(4, 2, 6);
-  }
+  if (tile_rows == 128) PICK(2, 2, 4);
+  PICK(4, 2, 4);
 #undef PICK
 #undef GO
 }

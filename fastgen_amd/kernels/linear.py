@@ -46,7 +46,6 @@ WIDE_ROWS = ops.SKINNY_MAX_ROWS  # the wide kernel (64 columns a workgroup): up 
 # the tiled kernel takes any number of rows; it is offered where it has been seen to win or come close (from the
 # wide kernel's range up to a few hundred rows; beyond, the library's large tiles are twice as fast)
 TILED_MIN_ROWS, TILED_MAX_ROWS = 65, 512
-TILED_TILES = ((0, 128), (2, 256))  # (config of ops.gemm_tiled, rows of its tile), both 128 columns wide
 
 
 def _aligned(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -228,7 +227,7 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         if rows <= WIDE_ROWS:
             candidates.append(("wide", lambda: ops.gemm_skinny(src, w, silu_mul_epilogue=True, wide=True)))
         if tiled_ok:
-            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, w, silu_mul_epilogue=True, config=TILED_TILES[1][0])))
+            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, w, silu_mul_epilogue=True, tile_rows=256)))
     elif own and not silu:
         if rows <= SKINNY_ROWS:
             candidates.append(("narrow", lambda: ops.gemm_skinny(src, w, out_dtype, wide=False)))
@@ -239,10 +238,10 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         elif rows <= 64:
             candidates.append(("wide", lambda: ops.gemm_skinny(x, w, out_dtype, wide=True)))
         if tiled_ok and partials_ok and out_dtype == torch.bfloat16:
-            for name, (config, tile_rows) in zip(("tiled", "tiled256"), TILED_TILES):
+            for name, tile_rows in zip(("tiled", "tiled256"), ops.TILED_TILE_ROWS):
                 s_t = tiled_splits(N, K, rows, tile_rows)
-                candidates.append((name, lambda config=config, s_t=s_t: ops.gemm_tiled(x, w, out_dtype, k_splits=s_t,
-                                                                                       config=config)))
+                candidates.append((name, lambda tile_rows=tile_rows, s_t=s_t: ops.gemm_tiled(
+                    x, w, out_dtype, k_splits=s_t, tile_rows=tile_rows)))
                 handicap[name] = sums_cost(s_t)
     if scaled is None or not candidates:
         candidates.append(("library", library))

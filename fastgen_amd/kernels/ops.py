@@ -616,15 +616,15 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     return y
 
 
-TILED_CONFIGS = 5
+TILED_TILE_ROWS = (128, 256)  # rows of x a workgroup of the tiled kernel takes (by 128 columns)
 
 
 def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-               silu_mul_epilogue: bool = False, k_splits: int = 1, config: int = 0) -> torch.Tensor:
+               silu_mul_epilogue: bool = False, k_splits: int = 1, tile_rows: int = 128) -> torch.Tensor:
     """``x @ w.T`` for many rows of bf16 ``x`` by the engine's tiled MFMA kernel (both operands through a
     ring of LDS stages), with the k range cut over workgroups if ``k_splits > 1``: the result is then
-    fp32 ``[k_splits, M, N]`` partial sums.  ``config`` picks the tile (128 or 256 rows by 128 or 256
-    columns) and the ring's depth.  With ``silu_mul_epilogue`` as :func:`gemm_skinny`."""
+    fp32 ``[k_splits, M, N]`` partial sums.  ``tile_rows``: 128 or 256 rows of x a workgroup (by 128
+    columns).  With ``silu_mul_epilogue`` as :func:`gemm_skinny`."""
     _gpu(x, w)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_tiled takes bfloat16 operands")
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
@@ -633,7 +633,7 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     _need(M > 0 and K % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
           and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
           "K must be a multiple of 8, rows 16-byte aligned")
-    _need(0 <= config < TILED_CONFIGS, f"config must be 0..{TILED_CONFIGS - 1}")
+    _need(tile_rows in TILED_TILE_ROWS, f"tile_rows must be one of {TILED_TILE_ROWS}")
     out_dtype = out_dtype or torch.bfloat16
     if silu_mul_epilogue:
         _need(N % 16 == 0 and out_dtype == torch.bfloat16 and k_splits == 1,
@@ -645,7 +645,7 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
     st = _lib.load("gemm_tiled").fg_gemm_tiled(
         _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N, K,
-        _code(y), 1 if silu_mul_epilogue else 0, int(config), _stream(x))
+        _code(y), 1 if silu_mul_epilogue else 0, int(tile_rows), _stream(x))
     _check(st, "gemm_tiled")
     return y
 

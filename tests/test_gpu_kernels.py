@@ -382,18 +382,18 @@ def test_gemm_skinny_wide_gate_up(ops, M):
     assert got.shape == (M, F) and (got.float() - want).abs().max() <= 1e-2 * want.abs().max() + 1e-3
 
 
-@pytest.mark.parametrize("config", range(5))
+@pytest.mark.parametrize("tile_rows", [128, 256])
 @pytest.mark.parametrize("M,N,K,S", [(129, 515, 240, 1), (192, 4096, 4096, 8), (256, 4096, 14336, 16), (1, 16, 8, 1),
                                      (300, 100, 264, 3), (2048, 256, 1000, 2), (65, 6144, 64, 2)])
-def test_gemm_tiled_and_k_splits(ops, config, M, N, K, S):
-    """The tiled product (both operands through a ring of LDS stages) at every tile shape: sizes that are no
+def test_gemm_tiled_and_k_splits(ops, tile_rows, M, N, K, S):
+    """The tiled product (both operands through a ring of LDS stages) at both tile shapes: sizes that are no
     multiple of a tile, of a stage (32 k) or of anything but 8; one row; k splits whose ranges are not equal;
     each split's partial sums against the product over its own k range."""
     torch.manual_seed(M + N)
     x = torch.randn(M, K).bfloat16()
     w = (torch.randn(N, K) * K**-0.5).bfloat16()
     want = x.double() @ w.double().T
-    got = ops.gemm_tiled(x.to(DEV), w.to(DEV), k_splits=S, config=config)
+    got = ops.gemm_tiled(x.to(DEV), w.to(DEV), k_splits=S, tile_rows=tile_rows)
     if S > 1:
         assert got.dtype == torch.float32 and got.shape == (S, M, N)
         step = -(-K // (S * 32)) * 32
@@ -404,7 +404,7 @@ def test_gemm_tiled_and_k_splits(ops, config, M, N, K, S):
     else:
         assert got.dtype == torch.bfloat16 and got.shape == (M, N)
     assert (got.cpu().double() - want).abs().max() <= (1e-4 if S > 1 else 1e-2) * want.abs().max() + 1e-6
-    y32 = ops.gemm_tiled(x.to(DEV), w.to(DEV), torch.float32, config=config)
+    y32 = ops.gemm_tiled(x.to(DEV), w.to(DEV), torch.float32, tile_rows=tile_rows)
     assert y32.dtype == torch.float32 and (y32.cpu().double() - want).abs().max() <= 1e-4 * want.abs().max() + 1e-6
 
 
@@ -416,8 +416,8 @@ def test_gemm_tiled_gate_up_epilogue(ops, M, F, K):
     w = ops.interleave_gate_up(wg, wu).contiguous().to(DEV)
     g, u = x.float() @ wg.float().T, x.float() @ wu.float().T
     want = g * torch.sigmoid(g) * u
-    for config in (0, 2, 3):
-        got = ops.gemm_tiled(x.to(DEV), w, silu_mul_epilogue=True, config=config).cpu().float()
+    for tile_rows in (128, 256):
+        got = ops.gemm_tiled(x.to(DEV), w, silu_mul_epilogue=True, tile_rows=tile_rows).cpu().float()
         assert got.shape == (M, F) and (got - want).abs().max() <= 1.5e-2 * want.abs().max() + 1e-3
 
 

@@ -314,11 +314,11 @@ def test_gemm_tiled_twins(ops, M, N, K):
     torch.manual_seed(N)
     bf = torch.bfloat16
     x, w = (torch.randn(M, K) / 4).to(bf), (torch.randn(N, K) / 4).to(bf)
-    for config in range(kernel_ops.TILED_CONFIGS):
-        _both("gemm_tiled", lambda: (x, w, None, False, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
-        _both("gemm_tiled", lambda: (x, w, torch.float32, False, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
-        _both("gemm_tiled", lambda: (x, w, None, True, 1, config), lambda g, t, *_: _close(g, t, bf), ops)
-        _both("gemm_tiled", lambda: (x, w, None, False, 3, config),
+    for tile_rows in kernel_ops.TILED_TILE_ROWS:
+        _both("gemm_tiled", lambda: (x, w, None, False, 1, tile_rows), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, torch.float32, False, 1, tile_rows), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, None, True, 1, tile_rows), lambda g, t, *_: _close(g, t, bf), ops)
+        _both("gemm_tiled", lambda: (x, w, None, False, 3, tile_rows),
               lambda g, t, *_: (_close(g.sum(0), t.sum(0), bf), torch.testing.assert_close(g.cpu(), t, rtol=2e-3, atol=2e-3)), ops)
 
 
