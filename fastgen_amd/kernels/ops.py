@@ -11,7 +11,7 @@ from __future__ import annotations
 import ctypes
 from dataclasses import dataclass
 import os
-from typing import Optional
+from typing import Dict, Optional
 
 import numpy as np
 
@@ -349,6 +349,19 @@ def attention_plan(items: torch.Tensor, n_items: int, max_chunks: int, head_dim:
     return plan
 
 
+_ONE_STREAM = bool(os.environ.get("FG_ONE_STREAM"))  # no kernel runs beside another
+_second: Dict[int, "torch.cuda.Stream"] = {}
+
+
+def _second_stream(device) -> "torch.cuda.Stream":
+    """A stream of the default priority beside the current one, one a device, made at first use."""
+    index = torch.device(device).index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _second:
+        _second[index] = torch.cuda.Stream(device)
+    return _second[index]
+
+
 def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                          block_table: torch.Tensor, small_items: Optional[torch.Tensor],
                          big_items: Optional[torch.Tensor], n_heads: int, scale: float, window: int = 0,
@@ -360,7 +373,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
     ``plan``: :func:`attention_plan` of the small items with this ``max_chunks``
     and ``window`` (made here if not given).  ``max_rows``: no small item has
     more rows (tokens times query heads per kv head) than this.  ``tile_rows``: the
-    rows the big items were cut for (:func:`attention_tile_rows`; default: the larger form's)."""
+    rows the big items were cut for (:func:`attention_tile_rows`; default: the larger form's).
+    With items of both kinds the tile kernel runs on a second stream beside the split kernel and
+    the current stream waits for it before this returns (not while a graph is captured, not with
+    ``FG_ONE_STREAM=1``)."""
     _gpu(q, out, k_pages, v_pages, block_table, small_items, big_items, plan)
     n_pages, n_kv, page_size, hd = k_pages.shape
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
@@ -378,6 +394,14 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
           "block_table must be int32 [B, max_pages]")
     lib = _lib.load(f"attention_mfma@{hd}")
     G = n_heads // n_kv
+    beside = None
+    if (small_items is not None and small_items.numel() and big_items is not None and big_items.numel()
+            and not _ONE_STREAM and not torch.cuda.is_current_stream_capturing()):
+        # a step with both kinds of items (prompt portions beside decoded tokens): the two kernels write
+        # different rows of `out`, one is bound by the matrix cores and one by memory, so the tile kernel
+        # runs on a second stream beside the split kernel (3 % of a continuous-batching run)
+        beside = _second_stream(q.device)
+        beside.wait_event(torch.cuda.current_stream(q.device).record_event())
     if small_items is not None and small_items.numel():
         _need(G <= 16 and 1 <= max_rows <= 16, "the split kernel takes at most 16 rows an item")
         _i32(small_items, "small_items")
@@ -406,8 +430,10 @@ def paged_attention_mfma(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tens
         st = lib.fg_attn_tile(
             _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.stride(0), _ptr(big_items), big_items.numel() // 4, tile_rows, n_heads, n_kv, hd, page_size,
-            ctypes.c_float(scale), int(window or 0), _stream(q))
+            ctypes.c_float(scale), int(window or 0), ctypes.c_void_p(beside.cuda_stream) if beside else _stream(q))
         _check(st, "attn_tile")
+        if beside is not None:
+            torch.cuda.current_stream(q.device).wait_event(beside.record_event())
     return out
 
 

@@ -707,6 +707,49 @@ def test_paged_attention_mfma(ops, H, KV, hd, P, window, cut):
     assert torch.allclose(out.cpu().float(), want, atol=1.5e-2, rtol=2e-2)
 
 
+def test_paged_attention_mfma_two_streams(ops, monkeypatch):
+    """Prompt portions beside decoded tokens: the tile kernel runs on a second stream beside the
+    split kernel.  The result is there when the caller's stream goes on (work queued behind the
+    call, on a stream that is not the default one, sees every row), equals the one-stream result
+    bit for bit, and a call while a graph is captured stays on the capturing stream."""
+    import numpy as np
+
+    H, KV, hd, P = 32, 8, 128, 64
+    seqs = [(900, 1), (0, 700), (2000, 1), (300, 260), (64, 1)]
+    case = _paged_case(torch.bfloat16, seqs, H, KV, hd, P, seed=26)
+    q_lens = [b for _, b in seqs]
+    small, big = ops.attention_items(q_lens, np.concatenate([[0], np.cumsum(q_lens)]), [a for a, _ in seqs], H // KV,
+                                     ops.attention_tile_rows(hd))
+    assert small.size and big.size
+    small, big = (torch.from_numpy(a.reshape(-1)).to(DEV) for a in (small, big))
+
+    def run(out):
+        return ops.paged_attention_mfma(case["q"], out, case["kp"], case["vp"], case["table"], small, big, H,
+                                        hd ** -0.5)
+
+    monkeypatch.setattr(ops, "_ONE_STREAM", True)
+    one = run(torch.full_like(case["q"], float("nan")))
+    assert torch.allclose(one.cpu().float(), _plain_rows(case, seqs), atol=1.5e-2, rtol=2e-2)
+    monkeypatch.setattr(ops, "_ONE_STREAM", False)
+    mine = torch.cuda.Stream(DEV)
+    mine.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(mine):
+        for _ in range(3):
+            two = run(torch.full_like(case["q"], float("nan")))
+            copy = two.clone()  # queued on the caller's stream right behind the call
+            mine.synchronize()
+            assert torch.equal(copy, one)
+    held = torch.empty_like(case["q"])
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run(held)
+    for _ in range(2):
+        held.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(held, one)
+
+
 @pytest.mark.parametrize("cut", ["coarse", "pairs", "fine"])
 def test_paged_attention_mfma_far_key_and_edges(ops, cut):
     """A key that gets nearly all the weight, at the edges of tiles, pages and
