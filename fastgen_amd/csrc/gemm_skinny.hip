@@ -14,11 +14,39 @@
 //    silu(gate) * up directly: the gate/up activations never reach memory.
 //
 // Replaces the library product of fastgen/forward.py:433-513 where M is small.
+//
+// W comes row by row (ldw = elements between rows), or packed (ldw = 0): in blocks of 16 rows x 32 k
+// of 1 KB, each in the order in which a wave's lanes hold an MFMA operand (lane 16 g + r: row r, k
+// 8 g .. 8 g + 7), the blocks of 16 rows one after the other along k, rows and k padded with zeros to
+// whole blocks: [ceil(N / 16)][ceil(K / 32)][64][8].  A wave's load of an operand is then 1 KB of
+// whole cache lines, and its eight loads of a pass 8 KB in a row; from rows it is 16 pieces of 64
+// bytes, half a cache line each, whose other halves the next load asks for again: the kernels here
+// are bound by the number of such requests, not by the bytes.
 #include "common.h"
 #include "kv_layout.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Where a lane finds its 16 bytes of W for the 16 rows from n0 on: at base + (k / 32) * step for the
+// k step of 32 that begins at k (a multiple of 32).  A lane whose chunk lies beyond the k range loads
+// `safe` instead (every load is issued, none is conditional) and zeroes what it got.
+struct WSrc {
+  const bf16_t* base;
+  const bf16_t* safe;
+  int step;
+  __device__ __forceinline__ const bf16x8* at(int k, bool in) const {
+    return (const bf16x8*)(in ? base + (size_t)(k >> 5) * step : safe);
+  }
+};
+__device__ __forceinline__ WSrc w_src(const bf16_t* w, int ldw, int n0, int N, int K, int lane) {
+  if (ldw) {  // rows are clamped, not skipped: what they give is not stored
+    const bf16_t* row = w + (size_t)min(n0 + (lane & 15), N - 1) * ldw;
+    return WSrc{row + 8 * (lane >> 4), row, 32};
+  }
+  const bf16_t* block = w + ((size_t)min(n0 >> 4, (N - 1) >> 4) * ((K + 31) >> 5) * 64 + lane) * 8;
+  return WSrc{block, block, 512};
+}
 
 #define EPI_STORE 0
 #define EPI_SILU_MUL 1
@@ -142,8 +170,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
-  // rows are clamped, not skipped: what they give is not stored
-  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const WSrc ws = w_src(w, ldw, n0, N, K, lane);
   const bf16_t* xrow[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) xrow[mb] = x + (size_t)min(16 * mb + r16, M - 1) * ldx;
@@ -162,7 +189,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
       const int k = kk + 32 * u + 8 * g;
       const bool in = k < k_end;  // K % 8 == 0: a chunk is inside or outside as a whole
       const int kc = in ? k : k_begin;
-      const bf16x8 av = *(const bf16x8*)(wrow + kc);
+      const bf16x8 av = *ws.at(kk + 32 * u, in);
       a[u] = in ? av : gs_zero8();
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) b[u][mb] = *(const bf16x8*)(xrow[mb] + kc);
@@ -231,7 +258,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
-  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const WSrc ws = w_src(w, ldw, n0, N, K, lane);
   const int kw = ((K + WAVES * 32 - 1) / (WAVES * 32)) * 32;
   const int k_begin = min(K, wave * kw), k_end = min(K, k_begin + kw);
   // copying x: a row's 256 k of one iteration are 32 chunks = 32 lanes; a load covers 2 rows
@@ -246,7 +273,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny16_kernel(
     for (int u = 0; u < U; ++u) {
       const int k = kk + 32 * u + 8 * g;
       const bool in = k < k_end;
-      const bf16x8 av = *(const bf16x8*)(wrow + (in ? k : k_begin));
+      const bf16x8 av = *ws.at(kk + 32 * u, in);
       a[u] = in ? av : gs_zero8();
     }
 #pragma unroll
@@ -366,7 +393,7 @@ __global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
   const int lane = threadIdx.x % FG_WAVE, wave = threadIdx.x / FG_WAVE;
   const int r16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 64 + wave * 16;
-  const bf16_t* wrow = w + (size_t)min(n0 + r16, N - 1) * ldw;
+  const WSrc ws = w_src(w, ldw, n0, N, K, lane);
   const int k_begin = min(K, (int)blockIdx.y * k_per_split), k_end = min(K, k_begin + k_per_split);
   f32x4 acc[MB];
 #pragma unroll
@@ -388,7 +415,7 @@ __global__ __launch_bounds__(256, MB <= 4 ? 3 : 2) void gemm_skinny64_kernel(
     for (int u = 0; u < U; ++u) {
       const int k = kk + 32 * u + 8 * g;
       const bool in = k < k_end;
-      const bf16x8 av = *(const bf16x8*)(wrow + (in ? k : k_begin));
+      const bf16x8 av = *ws.at(kk + 32 * u, in);
       a_next[u] = in ? av : gs_zero8();
     }
   };
@@ -462,13 +489,14 @@ static void launch_skinny(const void* x, int ldx, const void* w, int ldw, void* 
                                                                    (TY*)y, ldy, M, N, K, sc, rs);
 }
 
-// x [M, K] bf16 (M <= 64), w [N, K] bf16, K % 8 == 0, rows 16-byte aligned.
+// x [M, K] bf16 (M <= 64), w [N, K] bf16, K % 8 == 0, rows 16-byte aligned; ldw = 0: w is packed (see the top;
+// so in every entry point of this file).
 // epilogue 0: y [M, N] of out_dtype; epilogue 1: w's rows interleaved gate/up in
 // groups of 8 (N % 16 == 0), y [M, N/2] = silu(gate) * up of out_dtype.
 extern "C" int fg_gemm_skinny(const void* x, int ldx, const void* w, int ldw, void* y, int ldy, int M, int N,
                               int K, int out_dtype, int epilogue, hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
-  if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return FG_ERR_ARG;
+  if (M > 64 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K)) return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && ldy < N) return FG_ERR_ARG;
   if (epilogue != EPI_STORE && epilogue != EPI_SILU_MUL) return FG_ERR_ARG;
@@ -504,7 +532,7 @@ extern "C" int fg_gemm_skinny_fused(const void* x, int ldx, const void* w, int l
                                     float* h, int ldh, const void* norm_w, int norm_w_dtype, void* x_out, int ldxo,
                                     float* ssq_out, hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
-  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K) return FG_ERR_ARG;
+  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K)) return FG_ERR_ARG;
   if (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))) return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || !y)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || !y)) return FG_ERR_ARG;
@@ -532,7 +560,7 @@ extern "C" int fg_gemm_skinny64(const void* x, int ldx, const void* w, int ldw, 
   if (M <= 0 || N <= 0) return FG_OK;
   if (ssq && (M > 16 || k_splits != 1 || n_parts < 1 || dim < 1 || !(eps >= 0.f))) return FG_ERR_ARG;
   const RowScale sc{ssq, n_parts, ssq ? 1.f / (float)dim : 0.f, eps};
-  if (M > 128 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535)
+  if (M > 128 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || k_splits < 1 || k_splits > 65535)
     return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;
   if (epilogue == EPI_STORE && (ldy < N || (k_splits > 1 && out_dtype != FG_F32))) return FG_ERR_ARG;
@@ -573,7 +601,7 @@ extern "C" int fg_gemm_skinny_qkv(const void* x, int ldx, const void* w, int ldw
                                   const float* ssq, int n_parts, int dim, float eps, hipStream_t stream) {
   if (M <= 0) return FG_OK;
   const int N = (n_heads + 2 * n_kv) * hd;
-  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || hd % 16 || n_heads <= 0 ||
+  if (M > 16 || K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || hd % 16 || n_heads <= 0 ||
       n_kv <= 0 || rotary_dim < 0 || rotary_dim > hd || rotary_dim % 2 || page_size <= 0 || page_size % 8 ||
       ldy < n_heads * hd || ldy % 2 || !slots || !k_pages || !v_pages || (rotary_dim && !table) ||
       (ssq && (n_parts < 1 || dim < 1 || !(eps >= 0.f))))

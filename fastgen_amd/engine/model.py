@@ -8,6 +8,7 @@ The reference's counterpart is the weight-only ``Transformer`` skeleton
 
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Dict, List, Mapping, Optional, Sequence
@@ -15,8 +16,10 @@ from typing import Any, Dict, List, Mapping, Optional, Sequence
 import torch
 
 from ..config import ModelLayout, PartSpec, get_architecture, read_config_json
+from ..kernels.linear import StreamedMatrix, packing, packing_fits
 from ..kernels.ops import ScaledRows
 from ..parts import LayerStore, PagedNeed, StateNeed, TensorSpec, build_part
+from ..parts.base import MATRIX
 from ..weights.source import RandomSource, SafetensorsSource, TensorSource, check_against_specs
 from .context import StepContext
 
@@ -60,45 +63,56 @@ def build_parts(layout: ModelLayout) -> ModelParts:
 
 class Model:
     def __init__(self, layout: ModelLayout, dtype: torch.dtype, device: torch.device | str, args: Any = None,
-                 architecture: Optional[str] = None) -> None:
+                 architecture: Optional[str] = None, packed_weights: Optional[bool] = None) -> None:
+        """``packed_weights``: whether the bfloat16 matrices get a second copy in the order in which the
+        products of few rows read them (``kernels.linear.StreamedMatrix``); None: if the weights twice
+        leave half of the GPU's memory free (``kernels.linear.packing_fits``)."""
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"dtype {dtype} is not supported (float32 or bfloat16)")
         self.layout, self.dtype, self.device = layout, dtype, torch.device(device)
         self.args, self.architecture = args, architecture
+        self.packed_weights = packed_weights
         self.parts = build_parts(layout)
         self.vocab_size = layout.vocab_size
         self.loaded = False
 
     # ------------------------------------------------------------- build
     @classmethod
-    def from_config(cls, config: Mapping[str, Any], dtype: torch.dtype, device: torch.device | str) -> "Model":
+    def from_config(cls, config: Mapping[str, Any], dtype: torch.dtype, device: torch.device | str,
+                    packed_weights: Optional[bool] = None) -> "Model":
         arch = get_architecture(config)
         args = arch.parse(config)
-        return cls(arch.layout(args), dtype, device, args=args, architecture=arch.name)
+        return cls(arch.layout(args), dtype, device, args=args, architecture=arch.name, packed_weights=packed_weights)
 
     @classmethod
-    def from_folder(cls, model_dir: str | Path, dtype: torch.dtype, device: torch.device | str) -> "Model":
+    def from_folder(cls, model_dir: str | Path, dtype: torch.dtype, device: torch.device | str,
+                    packed_weights: Optional[bool] = None) -> "Model":
         """The model that ``config.json`` names, with the folder's weights."""
-        model = cls.from_config(read_config_json(model_dir), dtype, device)
+        model = cls.from_config(read_config_json(model_dir), dtype, device, packed_weights)
         model.load(SafetensorsSource(model_dir))
         return model
 
     @classmethod
     def random(cls, config: Mapping[str, Any], seed: int, dtype: torch.dtype,
-               device: torch.device | str) -> "Model":
+               device: torch.device | str, packed_weights: Optional[bool] = None) -> "Model":
         """Seeded random weights drawn on the device, without a folder."""
-        model = cls.from_config(config, dtype, device)
+        model = cls.from_config(config, dtype, device, packed_weights)
         model.load(RandomSource(model.parts.tensor_specs(), seed, dtype, device))
         return model
 
     def load(self, source: TensorSource) -> None:
         specs = self.parts.tensor_specs()
         check_against_specs(source, specs, self.parts.duplicates())
-        for part in self.parts.all_parts:
-            tensors = {s.name: source.get(s.name) for s in part.tensor_specs()}
-            part.load(tensors, self.dtype, self.device)
-        if getattr(self.parts.head, "tied_to", None):
-            self.parts.head.tie(self.parts.embed.weight)
+        pack = self.packed_weights
+        if pack is None:
+            matrix_bytes = sum(math.prod(s.shape) for s in specs if s.role == MATRIX) * 2
+            pack = self.dtype == torch.bfloat16 and packing_fits(matrix_bytes, self.device)
+        with packing(pack and self.dtype == torch.bfloat16):
+            for part in self.parts.all_parts:
+                tensors = {s.name: source.get(s.name) for s in part.tensor_specs()}
+                part.load(tensors, self.dtype, self.device)
+            if getattr(self.parts.head, "tied_to", None):
+                self.parts.head.tie(self.parts.embed.weight)
         self.loaded = True
 
     # ------------------------------------------------------------- needs
@@ -125,9 +139,11 @@ class Model:
         seen, total = set(), 0
         for p in self.parts.all_parts:
             for v in vars(p).values():
-                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
-                    seen.add(v.data_ptr())
-                    total += v.numel() * v.element_size()
+                held = [v.rows, v.packed.data if v.packed is not None else None] if isinstance(v, StreamedMatrix) else [v]
+                for t in held:
+                    if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                        seen.add(t.data_ptr())
+                        total += t.numel() * t.element_size()
         return total
 
     # ------------------------------------------------------------- forward

@@ -11,7 +11,7 @@ from __future__ import annotations
 import ctypes
 from dataclasses import dataclass
 import os
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import numpy as np
 
@@ -514,6 +514,68 @@ SKINNY_MAX_ROWS = 128
 
 
 @dataclass
+class PackedWeight:
+    """A bfloat16 weight matrix ``[n, k]`` in the order in which the streaming products read it
+    (:func:`pack_weight`): ``data [ceil(n / 16), ceil(k / 32), 64, 8]``, a block of 16 rows x 32 k as
+    the 1 KB that a wave holds as one MFMA operand (lane ``16 g + r``: row ``r``, k ``8 g .. 8 g + 7``),
+    rows and k padded with zeros.  A wave's load is then whole cache lines in a row; from a matrix
+    stored row by row it is 16 pieces of half a line."""
+
+    data: torch.Tensor
+    n: int
+    k: int
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return (self.n, self.k)
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.data.dtype
+
+    def first_rows(self, n: int) -> "PackedWeight":
+        """The matrix of the first ``n`` rows (a multiple of 16, or all): a view."""
+        _need(0 < n <= self.n and (n % 16 == 0 or n == self.n), "a packed matrix is cut at multiples of 16 rows")
+        return PackedWeight(self.data[: -(-n // 16)], n, self.k)
+
+
+def pack_weight(w: torch.Tensor) -> PackedWeight:
+    """``w [n, k]`` (bfloat16) as :class:`PackedWeight`: a copy, on the device of ``w``."""
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16, "pack_weight takes a bfloat16 matrix")
+    n, k = w.shape
+    nb, ks = -(-n // 16), -(-k // 32)
+    if (nb * 16, ks * 32) != (n, k):
+        padded = w.new_zeros((nb * 16, ks * 32))
+        padded[:n, :k] = w
+        w = padded
+    # [nb, r, ks, g, 8] -> [nb, ks, g, r, 8]
+    data = w.view(nb, 16, ks, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(nb, ks, 64, 8)
+    return PackedWeight(data, n, k)
+
+
+def unpack_weight(p: PackedWeight) -> torch.Tensor:
+    """The matrix ``[n, k]`` that :func:`pack_weight` was given."""
+    nb, ks = p.data.shape[:2]
+    w = p.data.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)
+    return w[: p.n, : p.k].contiguous()
+
+
+def _weight_args(w, K: int, what: str):
+    """C arguments (pointer, ldw) for the weight of a streaming product, a matrix or :class:`PackedWeight`
+    (ldw = 0), checked against the k of x."""
+    if isinstance(w, PackedWeight):
+        _gpu(w.data)
+        _need(w.data.dtype == torch.bfloat16 and w.data.is_contiguous() and w.k == K
+              and w.data.shape == (-(-w.n // 16), -(-w.k // 32), 64, 8) and w.data.data_ptr() % 16 == 0,
+              f"{what}: the packed weight does not fit x [M, {K}]")
+        return _ptr(w.data), 0
+    _gpu(w)
+    _need(w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[1] == K, f"{what}: w must be bfloat16 [N, {K}]")
+    _need(w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0, f"{what}: w needs 16-byte aligned rows")
+    return _ptr(w), w.stride(0)
+
+
+@dataclass
 class ScaledRows:
     """Rows that are not yet divided by their root mean square: the true row ``t`` is
     ``rows[t] * rsqrt(sum(ssq[t]) / dim + eps)``.  For few rows the norm before a matrix product
@@ -558,19 +620,20 @@ def scale_rows(rows: torch.Tensor, ssq: torch.Tensor, dim: int, eps: float) -> t
     return out
 
 
-def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, h: torch.Tensor, norm_weight: torch.Tensor,
+def gemm_skinny_residual(x: torch.Tensor, w, h: torch.Tensor, norm_weight: torch.Tensor,
                          eps: float) -> ScaledRows:
     """For at most 16 rows: ``h += x @ w.T`` on the fp32 residual stream ``h [M, N]`` and, in the same
     kernel, what the RMSNorm that follows needs: ``h * norm_weight`` in bfloat16 and a sum of squares
-    of ``h`` per row and workgroup (16 columns).  ``x`` may itself be :class:`ScaledRows`."""
+    of ``h`` per row and workgroup (16 columns).  ``x`` may itself be :class:`ScaledRows`, ``w`` a
+    matrix or :class:`PackedWeight`."""
     rows = x.rows if isinstance(x, ScaledRows) else x
-    _gpu(rows, w, h, norm_weight)
+    _gpu(rows, h, norm_weight)
     M, K = rows.shape
     N = w.shape[0]
-    _need(rows.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] == K and 0 < M <= 16,
-          "gemm_skinny_residual takes bfloat16 x [M<=16, K] and w [N, K]")
-    _need(K % 8 == 0 and rows.stride(1) == 1 and w.stride(1) == 1 and rows.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-          and rows.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "K must be a multiple of 8, rows 16-byte aligned")
+    _need(rows.dtype == torch.bfloat16 and 0 < M <= 16, "gemm_skinny_residual takes bfloat16 x [M<=16, K] and w [N, K]")
+    _need(K % 8 == 0 and rows.stride(1) == 1 and rows.stride(0) % 8 == 0 and rows.data_ptr() % 16 == 0,
+          "K must be a multiple of 8, rows 16-byte aligned")
+    w_ptr, ldw = _weight_args(w, K, "gemm_skinny_residual")
     _need(h.dtype == torch.float32 and h.shape == (M, N) and h.stride(1) == 1, "h must be float32 [M, N]")
     _need(norm_weight.shape == (N,) and norm_weight.is_contiguous()
           and norm_weight.dtype in (torch.float32, torch.bfloat16), "norm_weight must be [N], float32 or bfloat16")
@@ -579,17 +642,17 @@ def gemm_skinny_residual(x: torch.Tensor, w: torch.Tensor, h: torch.Tensor, norm
     ssq_out = torch.empty((M, n_parts), dtype=torch.float32, device=rows.device)
     sc = _row_scale_args(x, M)
     st = _lib.load("gemm_skinny").fg_gemm_skinny_fused(
-        _ptr(rows), rows.stride(0), _ptr(w), w.stride(0), ctypes.c_void_p(0), 0, M, N, K, 3, *sc,
+        _ptr(rows), rows.stride(0), w_ptr, ldw, ctypes.c_void_p(0), 0, M, N, K, 3, *sc,
         _ptr(h), h.stride(0), _ptr(norm_weight), _code(norm_weight), _ptr(x_out), x_out.stride(0), _ptr(ssq_out),
         _stream(rows))
     _check(st, "gemm_skinny_residual")
     return ScaledRows(x_out, ssq_out, N, float(eps))
 
 
-def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None,
                 silu_mul_epilogue: bool = False, k_splits: int = 1, wide: Optional[bool] = None) -> torch.Tensor:
     """``x @ w.T`` for at most 128 rows of bf16 ``x`` on the matrix cores, built to
-    stream ``w [N, K]`` once.  ``x`` may be :class:`ScaledRows` (at most 16 rows, bfloat16 out): the
+    stream ``w [N, K]`` (a matrix or :class:`PackedWeight`) once.  ``x`` may be :class:`ScaledRows` (at most 16 rows, bfloat16 out): the
     result rows are scaled.  With ``silu_mul_epilogue`` ``w`` is a gate/up matrix
     ordered by :func:`interleave_gate_up` and the result is ``silu(gate) * up``
     ``[M, N/2]``.  With ``k_splits > 1`` the k range is cut over workgroups and the
@@ -600,14 +663,14 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     scaled = x if isinstance(x, ScaledRows) else None
     if scaled is not None:
         x = scaled.rows
-    _gpu(x, w)
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16 operands")
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
+    _gpu(x)
+    _need(x.dtype == torch.bfloat16 and x.dim() == 2, "gemm_skinny takes bfloat16 x [M, K]")
     M, K = x.shape
     N = w.shape[0]
     _need(0 < M <= SKINNY_MAX_ROWS, f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows, got {M}")
-    _need(K % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-          and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "K must be a multiple of 8, rows 16-byte aligned")
+    _need(K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
+          "K must be a multiple of 8, rows 16-byte aligned")
+    w_ptr, ldw = _weight_args(w, K, "gemm_skinny")
     out_dtype = out_dtype or torch.bfloat16
     if silu_mul_epilogue:
         _need(N % 16 == 0 and out_dtype == torch.bfloat16, "the gate/up epilogue needs N % 16 == 0 and bf16 output")
@@ -622,21 +685,21 @@ def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     if scaled is not None and wide:
         _need(M <= 16 and k_splits == 1 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
         st = lib.fg_gemm_skinny64(
-            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), 1, M, N,
+            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), 1, M, N,
             K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(scaled, M), _stream(x))
     elif scaled is not None:
         _need(M <= 16 and out_dtype == torch.bfloat16, "scaled rows: at most 16 rows, bfloat16 out")
         st = lib.fg_gemm_skinny_fused(
-            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, 1 if silu_mul_epilogue else 0,
+            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), y.stride(0), M, N, K, 1 if silu_mul_epilogue else 0,
             *_row_scale_args(scaled, M), ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0, ctypes.c_void_p(0), 0,
             ctypes.c_void_p(0), _stream(x))
     elif wide:
         st = lib.fg_gemm_skinny64(
-            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
+            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N,
             K, _code(y), 1 if silu_mul_epilogue else 0, *_row_scale_args(None, M), _stream(x))
     else:
         st = lib.fg_gemm_skinny(
-            _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), y.stride(0), M, N, K, _code(y),
+            _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), y.stride(0), M, N, K, _code(y),
             1 if silu_mul_epilogue else 0, _stream(x))
     _check(st, "gemm_skinny")
     return y
@@ -676,23 +739,24 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     return y
 
 
-def gemm_skinny_qkv(x, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots: torch.Tensor,
+def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor,
                     k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                     rotary_dim: int) -> torch.Tensor:
     """The q, k, v projections of at most 16 rows with :func:`rope_kv_write` in
     the product's epilogue: returns the rotated queries ``[M, H*hd]``; the rotated
-    keys and the values go straight into their cache pages.  ``x`` may be :class:`ScaledRows`."""
+    keys and the values go straight into their cache pages.  ``x`` may be :class:`ScaledRows`, ``wqkv`` a
+    matrix or :class:`PackedWeight`."""
     scaled = x if isinstance(x, ScaledRows) else None
     if scaled is not None:
         x = scaled.rows
-    _gpu(x, wqkv, table, slots, k_pages, v_pages)
-    _need(x.dim() == 2 and wqkv.dim() == 2 and k_pages.dim() == 4, "x [M, K], wqkv [N, K], k_pages [n, KV, P, hd]")
+    _gpu(x, table, slots, k_pages, v_pages)
+    _need(x.dim() == 2 and k_pages.dim() == 4, "x [M, K], wqkv [N, K], k_pages [n, KV, P, hd]")
     M, K = x.shape
-    _need(x.dtype == torch.bfloat16 and wqkv.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16
-          and v_pages.dtype == torch.bfloat16, "gemm_skinny_qkv takes bfloat16")
-    _need(0 < M <= 16 and wqkv.shape == ((n_heads + 2 * n_kv) * head_dim, K), "x [M<=16, K], wqkv [(H+2KV)*hd, K]")
-    _need(K % 8 == 0 and x.stride(1) == 1 and wqkv.stride(1) == 1 and x.stride(0) % 8 == 0
-          and wqkv.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and wqkv.data_ptr() % 16 == 0,
+    _need(x.dtype == torch.bfloat16 and k_pages.dtype == torch.bfloat16 and v_pages.dtype == torch.bfloat16,
+          "gemm_skinny_qkv takes bfloat16")
+    w_ptr, ldw = _weight_args(wqkv, K, "gemm_skinny_qkv")
+    _need(0 < M <= 16 and tuple(wqkv.shape) == ((n_heads + 2 * n_kv) * head_dim, K), "x [M<=16, K], wqkv [(H+2KV)*hd, K]")
+    _need(K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
           "K must be a multiple of 8, rows 16-byte aligned")
     _need(head_dim % 16 == 0, "head size must be a multiple of 16")
     page_size = k_pages.shape[2]
@@ -704,7 +768,7 @@ def gemm_skinny_qkv(x, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots:
               and table.shape == (M, rotary_dim // 2, 2), "table must be float32 [M, rotary_dim/2, 2]")
     q = torch.empty((M, n_heads * head_dim), dtype=torch.bfloat16, device=x.device)
     st = _lib.load("gemm_skinny").fg_gemm_skinny_qkv(
-        _ptr(x), x.stride(0), _ptr(wqkv), wqkv.stride(0), _ptr(q), q.stride(0), M, K,
+        _ptr(x), x.stride(0), w_ptr, ldw, _ptr(q), q.stride(0), M, K,
         _ptr(table if rotary_dim else None), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_heads, n_kv, head_dim,
         rotary_dim, page_size, *_row_scale_args(scaled, M), _stream(x))
     _check(st, "gemm_skinny_qkv")

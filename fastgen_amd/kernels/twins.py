@@ -18,7 +18,7 @@ from typing import Optional
 import torch
 
 from ..cache.layout import store_k, store_v, unpack_k, unpack_v
-from .ops import ScaledRows
+from .ops import PackedWeight, ScaledRows
 
 
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -192,16 +192,30 @@ def _rows(x) -> torch.Tensor:
     return x.float()
 
 
+def _matrix(w) -> torch.Tensor:
+    """The weight matrix ``[N, K]`` in fp32, from a matrix or from :class:`PackedWeight` (the inverse of the
+    packing, written out: block ``[nb, ks]`` holds rows ``16 nb + r`` and k ``32 ks + 8 g + e`` at lane
+    ``16 g + r``, element ``e``)."""
+    if not isinstance(w, PackedWeight):
+        return w.float()
+    nb, ks = w.data.shape[:2]
+    out = torch.zeros((nb * 16, ks * 32), dtype=torch.float32, device=w.data.device)
+    for g in range(4):
+        for r in range(16):
+            out[r::16].view(nb, ks, 32)[:, :, 8 * g : 8 * g + 8] = w.data[:, :, 16 * g + r, :].float()
+    return out[: w.n, : w.k]
+
+
 def scale_rows(rows: torch.Tensor, ssq: torch.Tensor, dim: int, eps: float) -> torch.Tensor:
     return (rows.float() * torch.rsqrt(ssq.sum(1, keepdim=True) / dim + eps)).to(rows.dtype)
 
 
-def gemm_skinny(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False,
+def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue: bool = False,
                 k_splits: int = 1, wide: Optional[bool] = None) -> torch.Tensor:
-    """``x @ w.T`` (``x`` may be :class:`ScaledRows`); with ``silu_mul_epilogue`` ``silu(gate) * up`` of a gate/up
+    """``x @ w.T`` (``x`` may be :class:`ScaledRows`, ``w`` :class:`PackedWeight`: so in all three); with ``silu_mul_epilogue`` ``silu(gate) * up`` of a gate/up
     matrix interleaved in turns of 8; with ``k_splits > 1`` fp32 ``[S, M, N]`` partial sums over the k ranges
     ``[s * ceil(K / S / 256) * 256, ...)``.  ``wide`` only picks a kernel."""
-    xf, wf = _rows(x), w.float()
+    xf, wf = _rows(x), _matrix(w)
     if k_splits > 1:
         K = wf.shape[1]
         step = -(-K // (k_splits * 256)) * 256
@@ -235,20 +249,20 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     return y.to(out_dtype or torch.bfloat16)
 
 
-def gemm_skinny_residual(x, w: torch.Tensor, h: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
+def gemm_skinny_residual(x, w, h: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> ScaledRows:
     """``h += x @ w.T``; returns what the RMSNorm after it needs: ``h * norm_weight`` in bfloat16 and the sums of
     squares of ``h`` over each block of 16 columns."""
-    h += _rows(x) @ w.float().T
+    h += _rows(x) @ _matrix(w).T
     M, N = h.shape
     sq = torch.nn.functional.pad(h * h, (0, -N % 16)).view(M, -1, 16).sum(-1)
     return ScaledRows((h * norm_weight.float()).to(torch.bfloat16), sq, N, float(eps))
 
 
-def gemm_skinny_qkv(x, wqkv: torch.Tensor, table: Optional[torch.Tensor], slots: torch.Tensor, k_pages: torch.Tensor,
+def gemm_skinny_qkv(x, wqkv, table: Optional[torch.Tensor], slots: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rotary_dim: int) -> torch.Tensor:
     """The q, k, v projections with :func:`rope_kv_write` on the fp32 sums: returns the rotated queries in
     bfloat16; the rotated keys and the values go into the pages."""
-    qkv = _rows(x) @ wqkv.float().T
+    qkv = _rows(x) @ _matrix(wqkv).T
     T, q_cols, kv_cols = qkv.shape[0], n_heads * head_dim, n_kv * head_dim
     q = _rotate(qkv[:, :q_cols].view(T, n_heads, head_dim), table, rotary_dim)
     k = _rotate(qkv[:, q_cols : q_cols + kv_cols].view(T, n_kv, head_dim), table, rotary_dim)

@@ -13,7 +13,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear, skinny_ok
+from ..kernels.linear import StreamedMatrix, linear, skinny_ok, streamed
 from .base import LayerStore, Mixer, PagedNeed, TensorSpec, build_part, place, register_part, MATRIX
 
 
@@ -37,8 +37,8 @@ class Attention(Mixer):
                 " kernels work in chunks of 8 head dimensions, up to 512"
             )
         self.position = build_part("position", o["position"])
-        self.wqkv: Optional[torch.Tensor] = None
-        self.wo: Optional[torch.Tensor] = None
+        self.wqkv: Optional[StreamedMatrix] = None
+        self.wo: Optional[StreamedMatrix] = None
         self.freqs: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -54,8 +54,8 @@ class Attention(Mixer):
         wq = self.position.arrange_rows(tensors[self._name("q_proj.weight")], self.n_heads)
         wk = self.position.arrange_rows(tensors[self._name("k_proj.weight")], self.n_kv_heads)
         wv = tensors[self._name("v_proj.weight")]
-        self.wqkv = place(torch.cat([wq, wk, wv], dim=0), MATRIX, dtype, device)
-        self.wo = place(tensors[self._name("o_proj.weight")], MATRIX, dtype, device)
+        self.wqkv = streamed(place(torch.cat([wq, wk, wv], dim=0), MATRIX, dtype, device))
+        self.wo = streamed(place(tensors[self._name("o_proj.weight")], MATRIX, dtype, device))
         self.freqs = self.position.frequencies_on(device)
 
     def paged_need(self) -> PagedNeed:
@@ -80,11 +80,11 @@ class Attention(Mixer):
             x = x.materialize()
         if store.owns and self.head_dim % 16 == 0 and skinny_ok(rows, self.wqkv):
             # few rows (decode): rotation and cache write happen where the product is stored
-            qkv = ops.gemm_skinny_qkv(x, self.wqkv, table, group.slots, store.k_pages, store.v_pages, self.n_heads,
+            qkv = ops.gemm_skinny_qkv(x, self.wqkv.streaming, table, group.slots, store.k_pages, store.v_pages, self.n_heads,
                                       self.n_kv_heads, self.head_dim, self.position.rotary_dim)
         else:
             # an entry that reads another entry's cache needs its queries only
-            qkv = linear(x, self.wqkv if store.owns else self.wqkv[:q_width])
+            qkv = linear(x, self.wqkv if store.owns else self.wqkv.first_rows(q_width))
             ops.rope_kv_write(
                 qkv, ctx.positions, self.freqs, group.slots, store.k_pages, store.v_pages,
                 self.n_heads, self.n_kv_heads, self.head_dim, self.position.rotary_dim, write_kv=store.owns,

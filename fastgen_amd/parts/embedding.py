@@ -7,7 +7,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear
+from ..kernels.linear import StreamedMatrix, linear, streamed
 from .base import MATRIX, Part, TensorSpec, place, register_part
 
 
@@ -43,7 +43,7 @@ class LMHead(Part):
         self.vocab_size = int(spec.options["vocab_size"])
         self.dim = int(spec.options["dim"])
         self.tied_to: Optional[str] = spec.options.get("tied_to")
-        self.weight: Optional[torch.Tensor] = None
+        self.weight: Optional[StreamedMatrix] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
         if self.tied_to:
@@ -56,10 +56,10 @@ class LMHead(Part):
 
     def load(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: Any) -> None:
         if not self.tied_to:
-            self.weight = place(tensors[self._name("weight")], MATRIX, dtype, device)
+            self.weight = streamed(place(tensors[self._name("weight")], MATRIX, dtype, device))
 
     def tie(self, table: torch.Tensor) -> None:
-        self.weight = table
+        self.weight = streamed(table)  # the table itself row by row; a packed copy of it if copies are made
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32)

@@ -11,7 +11,7 @@ from typing import Any, List, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from ..kernels.linear import linear
+from ..kernels.linear import StreamedMatrix, linear, streamed
 from .base import MATRIX, FeedForward, TensorSpec, place, register_part
 
 
@@ -22,8 +22,8 @@ class SwiGLU(FeedForward):
         super().__init__(spec)
         self.dim = int(spec.options["dim"])
         self.hidden_dim = int(spec.options["hidden_dim"])
-        self.w_gate_up: Optional[torch.Tensor] = None
-        self.w_down: Optional[torch.Tensor] = None
+        self.w_gate_up: Optional[StreamedMatrix] = None
+        self.w_down: Optional[StreamedMatrix] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [
@@ -42,8 +42,8 @@ class SwiGLU(FeedForward):
             gate = torch.cat([gate, gate.new_zeros(pad, self.dim)])
             up = torch.cat([up, up.new_zeros(pad, self.dim)])
             down = torch.cat([down, down.new_zeros(self.dim, pad)], dim=1)
-        self.w_gate_up = place(ops.interleave_gate_up(gate, up), MATRIX, dtype, device)
-        self.w_down = place(down, MATRIX, dtype, device)
+        self.w_gate_up = streamed(place(ops.interleave_gate_up(gate, up), MATRIX, dtype, device))
+        self.w_down = streamed(place(down, MATRIX, dtype, device))
 
     def forward(self, x, then=None):
         """``x``: the normed rows, or ``ScaledRows`` (the gate/up product finishes the norm).  ``then``:

@@ -282,17 +282,21 @@ def test_many_requests_decode_together_bfloat16(n_live, captured, tmp_path):
                  plain_logits(weights, cfg, tokens, torch.bfloat16), f"{n_live} live")
 
 
-@pytest.mark.parametrize("forced", ["narrow", "wide", "tiled", "tiled256", "library", None])
-def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, tmp_path, monkeypatch):
+@pytest.mark.parametrize("forced,packed", [("narrow", True), ("narrow", False), ("wide", True), ("wide", False),
+                                           ("tiled", True), ("tiled256", False), ("library", True), (None, True),
+                                           (None, False)])
+def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, packed, tmp_path, monkeypatch):
     """Which kernel takes a matrix product is measured at run time (``fastgen_amd.kernels.linear``), so which
     one an engine test meets depends on the machine.  Here the engine runs once under each kernel's name
     (taken wherever it is among the candidates of a product) and once as measured: whole prompts (up to 150
     rows), mixed steps, and 20 requests decoding together (17..32 rows), every position against the plain
-    implementation."""
+    implementation.  ``packed``: with and without the second copy of the matrices in the streaming kernels'
+    order (a model too large for two copies runs without)."""
     from fastgen_amd.kernels import linear
 
     monkeypatch.setattr(linear, "force", forced)
     monkeypatch.setattr(linear, "choices", {})
+    monkeypatch.setenv("FG_PACKED_WEIGHTS", "1" if packed else "0")
     cfg = TINY_B
     weights = sharpen(plain_random_weights(cfg, 9))
     weights = {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
@@ -303,6 +307,10 @@ def test_every_kernel_that_may_be_chosen_gives_the_plain_logits(forced, tmp_path
     want, noise = plain_logits(weights, cfg, tokens), plain_logits(weights, cfg, tokens, torch.bfloat16)
     for name, trace in (("whole", traces.whole(lengths)), ("mixed", traces.mixed(lengths, seed=3))):
         runner = make_runner(folder, torch.bfloat16, 32, traces.max_live_tokens(trace, 64))
+        from fastgen_amd.kernels.linear import StreamedMatrix
+
+        held = [v for p in runner.model.parts.all_parts for v in vars(p).values() if isinstance(v, StreamedMatrix)]
+        assert len(held) == 4 * cfg["num_hidden_layers"] + 1 and all((m.packed is not None) == packed for m in held)
         got = run_trace(runner, trace, tokens)
         assert_close(got, want, torch.bfloat16, noise, f"forced {forced}, {name}")
     prompts = {f"r{i}": 5 + 3 * i for i in range(20)}

@@ -439,6 +439,68 @@ def test_gemm_skinny_takes_views_and_refuses_the_rest(ops):
                         torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV))
 
 
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 40, 64, 100, 128])
+@pytest.mark.parametrize("N,K", [(515, 240), (4096, 4096), (48, 8), (1008, 14336), (16, 328), (200, 72)])
+def test_streaming_products_read_a_packed_weight(ops, M, N, K):
+    """The weight in the order of the kernels' reads (``pack_weight``: blocks of 16 rows x 32 k, padded with
+    zeros) instead of row by row: only where a lane finds its bytes differs, so every product gives the same
+    bits.  Sizes that are no multiples of the blocks; every entry point that streams a weight."""
+    torch.manual_seed(M + N + K)
+    x = torch.randn(M, K).bfloat16().to(DEV)
+    w = (torch.randn(N, K) * K**-0.5).bfloat16().to(DEV)
+    pw = ops.pack_weight(w)
+    assert pw.data.shape == (-(-N // 16), -(-K // 32), 64, 8) and torch.equal(ops.unpack_weight(pw), w)
+    both = lambda fn: (fn(w), fn(pw))
+    if M <= 64:
+        for odtype in (torch.bfloat16, torch.float32):
+            a, b = both(lambda m: ops.gemm_skinny(x, m, out_dtype=odtype, wide=False))
+            assert torch.equal(a, b)
+        want = x.double() @ w.double().T
+        assert (b.double() - want).abs().max() / want.abs().max() < 1e-5
+    a, b = both(lambda m: ops.gemm_skinny(x, m, wide=True))
+    assert torch.equal(a, b)
+    for S in (2, 5):
+        a, b = both(lambda m: ops.gemm_skinny(x, m, k_splits=S, wide=True))
+        assert torch.equal(a, b)
+    if N % 16 == 0:
+        for wide in ([False] if M <= 64 else []) + [True]:
+            a, b = both(lambda m: ops.gemm_skinny(x, m, silu_mul_epilogue=True, wide=wide))
+            assert torch.equal(a, b)
+    if M <= 16:
+        nw = (1 + 0.1 * torch.randn(N)).to(DEV)
+        h0 = torch.randn(M, N, device=DEV)
+        ha, hb = h0.clone(), h0.clone()
+        sa, sb = ops.gemm_skinny_residual(x, w, ha, nw, 1e-5), ops.gemm_skinny_residual(x, pw, hb, nw, 1e-5)
+        assert torch.equal(ha, hb) and torch.equal(sa.rows, sb.rows) and torch.equal(sa.ssq, sb.ssq)
+        # a consumer of rows whose norm is still open (K of the next product = this N)
+        if N % 8 == 0:
+            w2 = (torch.randn(104, N) * N**-0.5).bfloat16().to(DEV)
+            pw2 = ops.pack_weight(w2)
+            for wide in (False, True):
+                assert torch.equal(ops.gemm_skinny(sa, w2, wide=wide), ops.gemm_skinny(sa, pw2, wide=wide))
+        # the first rows of a packed matrix, as an entry that reads another's cache takes its queries' rows
+        if N > 32:
+            assert torch.equal(ops.gemm_skinny(x, w[:32], wide=False), ops.gemm_skinny(x, pw.first_rows(32), wide=False))
+
+
+@pytest.mark.parametrize("M", [1, 7, 16])
+def test_gemm_skinny_qkv_reads_a_packed_weight(ops, M):
+    H, KV, hd, rot, P, K = 5, 1, 48, 48, 32, 240
+    torch.manual_seed(M)
+    x = (torch.randn(M, K) * 0.5).bfloat16().to(DEV)
+    w = (torch.randn((H + 2 * KV) * hd, K) * K**-0.5).bfloat16().to(DEV)
+    pos = torch.randint(0, 5000, (M,), dtype=torch.int32, device=DEV)
+    table = ops.rope_table(pos, plain_rope_frequencies(rot, 10000.0).to(DEV))
+    slots = torch.randperm(5 * P)[:M].to(torch.int32).to(DEV)
+    got = []
+    for m in (w, ops.pack_weight(w)):
+        kp = torch.full((5, KV, P, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+        vp = torch.full((5, KV, hd, P), 7.0, dtype=torch.bfloat16, device=DEV)
+        got.append((ops.gemm_skinny_qkv(x, m, table, slots, kp, vp, H, KV, hd, rot), kp, vp))
+    for a, b in zip(*got):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("M", [1, 8, 40])
 @pytest.mark.parametrize("F,K", [(328, 240), (14336, 4096), (8, 64)])
 def test_gemm_skinny_gate_up_epilogue(ops, M, F, K):
