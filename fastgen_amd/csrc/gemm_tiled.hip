@@ -75,9 +75,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(
 #pragma unroll
   for (int j = 0; j < LPW; ++j) {
     const int b = wave + NW * j;
-    src[j] = b < WB ? w + (size_t)min(n_base + 16 * b + r16, N - 1) * ldw + 8 * g
-                    : x + (size_t)min(m_base + 16 * (b - WB) + r16, M - 1) * ldx + 8 * g;
+    if (b >= WB) src[j] = x + (size_t)min(m_base + 16 * (b - WB) + r16, M - 1) * ldx + 8 * g;
+    else if (ldw) src[j] = w + (size_t)min(n_base + 16 * b + r16, N - 1) * ldw + 8 * g;
+    else src[j] = w + ((size_t)min((n_base >> 4) + b, (N - 1) >> 4) * ((K + 31) >> 5) * 64 + lane) * 8;  // packed
   }
+  // elements from one k step of 32 to the next: 32 along a row, 512 (a block) in a packed W
+  int step[LPW];
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) step[j] = (wave + NW * j < WB && !ldw) ? 16 : 1;
   // stage s into slot s % NST; beyond the last stage the last one again, which nobody reads (every
   // wave issues LPW loads a stage to the end, so the count it waits for stays the same)
   auto issue = [&](int s) {
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(
     bf16_t* slot = ring + (size_t)(s % NST) * NB * BLOCK;
 #pragma unroll
     for (int j = 0; j < LPW; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + koff),
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + (size_t)koff * step[j]),
                                        (__attribute__((address_space(3))) void*)(slot + (wave + NW * j) * BLOCK), 16, 0, 0);
   };
 
@@ -199,7 +204,8 @@ static int launch_tiled(const void* x, int ldx, const void* w, int ldw, void* y,
   return fg_launch_status();
 }
 
-// x [M, K] bf16, w [N, K] bf16, K % 8 == 0, rows 16-byte aligned.
+// x [M, K] bf16, w [N, K] bf16, K % 8 == 0, rows 16-byte aligned; ldw = 0: w is packed in blocks of 16 rows x 32 k
+// (gemm_skinny.hip), each of which is one block of a stage here and one contiguous KB in memory.
 // epilogue 0: y [M, N] of out_dtype (k_splits > 1: fp32 [k_splits, M, N], part_stride elements apart,
 // partial sums over K for the consumer to add in split order; a split's k range is a multiple of 32);
 // epilogue 1: w's rows are gate/up interleaved in groups of 8 (N % 16 == 0), y [M, N / 2] bf16 =
@@ -208,7 +214,7 @@ extern "C" int fg_gemm_tiled(const void* x, int ldx, const void* w, int ldw, voi
                              int k_splits, int M, int N, int K, int out_dtype, int epilogue, int tile_rows,
                              hipStream_t stream) {
   if (M <= 0 || N <= 0) return FG_OK;
-  if (K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || ldw < K || k_splits < 1 || k_splits > 65535 ||
+  if (K <= 0 || K % 8 || ldx % 8 || ldw % 8 || ldx < K || (ldw && ldw < K) || k_splits < 1 || k_splits > 65535 ||
       (tile_rows != 128 && tile_rows != 256))
     return FG_ERR_ARG;
   if (epilogue == EPI_SILU_MUL && (N % 16 || ldy < N / 2 || k_splits != 1 || out_dtype != FG_BF16)) return FG_ERR_ARG;

@@ -47,8 +47,9 @@ def step_memory_estimate(model: Model, max_step_tokens: int, max_batch: int) -> 
     widest = model.layout.dim
     for part in model.parts.all_parts[1:-1]:  # the layers' parts; the embedding and the head are not per token
         for v in vars(part).values():
-            if isinstance(v, torch.Tensor) and v.dim() == 2:
-                widest = max(widest, v.shape[0])
+            shape = getattr(v, "shape", None)  # a tensor or a kernels.linear.StreamedMatrix
+            if shape is not None and len(shape) == 2:
+                widest = max(widest, shape[0])
     return int(max_step_tokens * 12 * widest + 3 * max_batch * model.vocab_size * 4)
 
 

@@ -307,7 +307,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
         if rows <= WIDE_ROWS:
             candidates.append(("wide", lambda: ops.gemm_skinny(src, sw, silu_mul_epilogue=True, wide=True)))
         if tiled_ok:
-            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, w, silu_mul_epilogue=True, tile_rows=256)))
+            candidates.append(("tiled256", lambda: ops.gemm_tiled(x, sw, silu_mul_epilogue=True, tile_rows=256)))
     elif own and not silu:
         if rows <= SKINNY_ROWS:
             candidates.append(("narrow", lambda: ops.gemm_skinny(src, sw, out_dtype, wide=False)))
@@ -321,7 +321,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None,
             for name, tile_rows in zip(("tiled", "tiled256"), ops.TILED_TILE_ROWS):
                 s_t = tiled_splits(N, K, rows, tile_rows)
                 candidates.append((name, lambda tile_rows=tile_rows, s_t=s_t: ops.gemm_tiled(
-                    x, w, out_dtype, k_splits=s_t, tile_rows=tile_rows)))
+                    x, sw, out_dtype, k_splits=s_t, tile_rows=tile_rows)))
                 handicap[name] = sums_cost(s_t)
     if scaled is None or not candidates:
         candidates.append(("library", library))

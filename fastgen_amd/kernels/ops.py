@@ -708,20 +708,19 @@ def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None,
 TILED_TILE_ROWS = (128, 256)  # rows of x a workgroup of the tiled kernel takes (by 128 columns)
 
 
-def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+def gemm_tiled(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None,
                silu_mul_epilogue: bool = False, k_splits: int = 1, tile_rows: int = 128) -> torch.Tensor:
     """``x @ w.T`` for many rows of bf16 ``x`` by the engine's tiled MFMA kernel (both operands through a
     ring of LDS stages), with the k range cut over workgroups if ``k_splits > 1``: the result is then
     fp32 ``[k_splits, M, N]`` partial sums.  ``tile_rows``: 128 or 256 rows of x a workgroup (by 128
-    columns).  With ``silu_mul_epilogue`` as :func:`gemm_skinny`."""
-    _gpu(x, w)
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_tiled takes bfloat16 operands")
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x [M,K] and w [N,K] must share K")
+    columns).  With ``silu_mul_epilogue`` as :func:`gemm_skinny`; ``w`` a matrix or :class:`PackedWeight`."""
+    _gpu(x)
+    _need(x.dtype == torch.bfloat16 and x.dim() == 2, "gemm_tiled takes bfloat16 x [M, K]")
     M, K = x.shape
     N = w.shape[0]
-    _need(M > 0 and K % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1 and x.stride(0) % 8 == 0
-          and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0,
+    _need(M > 0 and K % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0,
           "K must be a multiple of 8, rows 16-byte aligned")
+    w_ptr, ldw = _weight_args(w, K, "gemm_tiled")
     _need(tile_rows in TILED_TILE_ROWS, f"tile_rows must be one of {TILED_TILE_ROWS}")
     out_dtype = out_dtype or torch.bfloat16
     if silu_mul_epilogue:
@@ -733,7 +732,7 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
     cols = N // 2 if silu_mul_epilogue else N
     y = torch.empty((k_splits, M, cols) if k_splits > 1 else (M, cols), dtype=out_dtype, device=x.device)
     st = _lib.load("gemm_tiled").fg_gemm_tiled(
-        _ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N, K,
+        _ptr(x), x.stride(0), w_ptr, ldw, _ptr(y), cols, ctypes.c_longlong(M * cols), k_splits, M, N, K,
         _code(y), 1 if silu_mul_epilogue else 0, int(tile_rows), _stream(x))
     _check(st, "gemm_tiled")
     return y

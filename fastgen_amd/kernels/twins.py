@@ -230,11 +230,11 @@ def gemm_skinny(x, w, out_dtype: Optional[torch.dtype] = None, silu_mul_epilogue
     return y.to(out_dtype or torch.bfloat16)
 
 
-def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+def gemm_tiled(x: torch.Tensor, w, out_dtype: Optional[torch.dtype] = None,
                silu_mul_epilogue: bool = False, k_splits: int = 1, tile_rows: int = 128) -> torch.Tensor:
     """``x @ w.T``; with ``silu_mul_epilogue`` as :func:`gemm_skinny`; with ``k_splits > 1`` fp32 ``[S, M, N]``
     partial sums over the k ranges ``[s * ceil(K / S / 32) * 32, ...)``.  ``tile_rows`` only picks a tile."""
-    xf, wf = x.float(), w.float()
+    xf, wf = x.float(), _matrix(w)
     if k_splits > 1:
         K = wf.shape[1]
         step = -(-K // (k_splits * 32)) * 32

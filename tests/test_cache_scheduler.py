@@ -618,3 +618,18 @@ def test_memory_budget_counts_the_per_request_state():
     assert with_state * per_token + state_bytes(needs, 999) + reserve <= free
     assert tokens_that_fit(free, groups, page, torch.bfloat16, reserve, needs, 999, at_most=100) == 96
     assert tokens_that_fit(free, groups, page, torch.bfloat16, reserve, needs, 10 ** 6) == 0  # the state alone is too much
+
+
+def test_step_memory_estimate_sees_the_widest_product():
+    """What a step's intermediate tensors may take is sized by the widest matrix of a layer (here the
+    gate/up matrix, 2 x 192 rows), whatever the part keeps its matrices in."""
+    import torch
+
+    from fastgen_amd.engine import Model
+    from fastgen_amd.engine.engine import step_memory_estimate
+    from plain_llama import TINY_A
+
+    model = Model.random(TINY_A, 0, torch.float32, "cpu")
+    widest = 2 * TINY_A["intermediate_size"]
+    assert widest > TINY_A["hidden_size"]
+    assert step_memory_estimate(model, 100, 4) == 100 * 12 * widest + 3 * 4 * TINY_A["vocab_size"] * 4

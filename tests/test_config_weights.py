@@ -189,6 +189,36 @@ def test_dtype_policy():
     assert place(torch.arange(4), TABLE_INT, torch.bfloat16, "cpu").dtype == torch.int32
 
 
+def test_second_copy_of_the_matrices_is_a_matter_of_memory(monkeypatch):
+    """``packing_fits``: the switch wins; without it nothing is packed off the GPU.  ``streamed`` packs only
+    while a model says so (``packing``), and only bfloat16 matrices on the GPU: the 32-bit path and a part
+    that hands ``linear`` a plain tensor keep one copy."""
+    from fastgen_amd.kernels import linear
+
+    monkeypatch.delenv("FG_PACKED_WEIGHTS", raising=False)
+    assert linear.packing_fits(1 << 30, "cpu") is False
+    monkeypatch.setenv("FG_PACKED_WEIGHTS", "1")
+    assert linear.packing_fits(1 << 50, "cpu") is True
+    monkeypatch.setenv("FG_PACKED_WEIGHTS", "0")
+    assert linear.packing_fits(1, "cpu") is False
+    w = torch.randn(48, 64).to(torch.bfloat16)
+    with linear.packing(True):
+        m = linear.streamed(w)  # on the CPU: one copy
+        assert m.packed is None and m.streaming is w and m.shape == w.shape and m.dtype == w.dtype
+    assert linear._pack_now is False
+    m = linear.StreamedMatrix(w, ops_pack(w))
+    assert m.streaming is m.packed and m.nbytes() == 2 * w.numel() * 2
+    cut = m.first_rows(32)
+    assert cut.rows.shape == (32, 64) and cut.packed is not None and cut.packed.shape == (32, 64)
+    assert m.first_rows(20).packed is None  # no multiple of 16: the rows alone
+
+
+def ops_pack(w):
+    from fastgen_amd.kernels import ops
+
+    return ops.pack_weight(w)
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py runs on one GPU: for more it says so in one line and exits with 2."""
     import subprocess

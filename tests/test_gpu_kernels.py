@@ -406,6 +406,11 @@ def test_gemm_tiled_and_k_splits(ops, tile_rows, M, N, K, S):
     assert (got.cpu().double() - want).abs().max() <= (1e-4 if S > 1 else 1e-2) * want.abs().max() + 1e-6
     y32 = ops.gemm_tiled(x.to(DEV), w.to(DEV), torch.float32, tile_rows=tile_rows)
     assert y32.dtype == torch.float32 and (y32.cpu().double() - want).abs().max() <= 1e-4 * want.abs().max() + 1e-6
+    # the weight packed in the kernels' blocks: the same bits
+    pw = ops.pack_weight(w.to(DEV))
+    assert torch.equal(ops.gemm_tiled(x.to(DEV), pw, torch.float32, tile_rows=tile_rows), y32)
+    assert torch.equal(ops.gemm_tiled(x.to(DEV), pw, k_splits=S, tile_rows=tile_rows),
+                       ops.gemm_tiled(x.to(DEV), w.to(DEV), k_splits=S, tile_rows=tile_rows))
 
 
 @pytest.mark.parametrize("M,F,K", [(129, 328, 240), (256, 14336, 4096), (70, 8, 64)])

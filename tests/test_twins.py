@@ -105,6 +105,31 @@ def test_rope_kv_write_twin_is_the_plain_rotation(H, KV, hd, rot, P):
     assert int((kn.abs().sum((1, 3)) > 0).sum()) == 8  # the token with slot -1 is written nowhere
 
 
+@pytest.mark.parametrize("N,K", [(16, 32), (37, 72), (515, 240), (64, 8)])
+def test_packed_weight_layout(N, K):
+    """``pack_weight`` against the layout written out element by element (the order the kernels' comment
+    gives: block ``[n / 16, k / 32]``, lane ``16 g + r`` holds row ``r`` and k ``8 g .. 8 g + 7``; rows and k
+    padded with zeros), its inverse, the twins' reading of it, and the cut at a multiple of 16 rows."""
+    torch.manual_seed(N)
+    w = torch.randn(N, K).to(torch.bfloat16)
+    p = kernel_ops.pack_weight(w)
+    nb, ks = -(-N // 16), -(-K // 32)
+    assert p.shape == (N, K) and p.data.shape == (nb, ks, 64, 8)
+    want = torch.zeros(nb, ks, 64, 8, dtype=torch.bfloat16)
+    for n in range(N):
+        for k in range(K):
+            want[n // 16, k // 32, 16 * ((k % 32) // 8) + n % 16, k % 8] = w[n, k]
+    assert torch.equal(p.data, want)
+    assert torch.equal(kernel_ops.unpack_weight(p), w)
+    assert torch.equal(twins._matrix(p), w.float())
+    x = torch.randn(3, K).to(torch.bfloat16)
+    assert torch.equal(twins.gemm_skinny(x, p), twins.gemm_skinny(x, w))
+    if N > 16:
+        assert torch.equal(kernel_ops.unpack_weight(p.first_rows(16)), w[:16])
+        with pytest.raises(kernel_ops.KernelArgumentError, match="multiples of 16"):
+            p.first_rows(17)
+
+
 def test_norm_twins_are_the_plain_norm():
     torch.manual_seed(5)
     h, d, w = torch.randn(7, 52), torch.randn(7, 52), torch.rand(52) + 0.5
