@@ -11,6 +11,10 @@ it is measured: the first time a product of some shape ``(N, K)`` meets some
 number of rows, the kernels that can take it are timed on the operands at hand
 (the caches emptied before each run) and the winner is kept in one table (``choices``) for every later product of
 that shape and row bucket.  No size of any model stands here or in the parts.
+
+A part hands ``linear`` its matrix as a :class:`StreamedMatrix` (made by :func:`streamed` when the part
+loads): the matrix row by row and, where a model's weights fit the GPU twice over, a second copy in the order
+in which the streaming kernels read it, which those kernels take.
 """
 
 from __future__ import annotations
