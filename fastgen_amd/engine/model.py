@@ -63,15 +63,17 @@ def build_parts(layout: ModelLayout) -> ModelParts:
 
 class Model:
     def __init__(self, layout: ModelLayout, dtype: torch.dtype, device: torch.device | str, args: Any = None,
-                 architecture: Optional[str] = None, packed_weights: Optional[bool] = None) -> None:
+                 architecture: Optional[str] = None, packed_weights: Optional[bool] = None,
+                 memory_budget: Optional[int] = None) -> None:
         """``packed_weights``: whether the bfloat16 matrices get a second copy in the order in which the
         products of few rows read them (``kernels.linear.StreamedMatrix``); None: if the weights twice
-        leave half of the GPU's memory free (``kernels.linear.packing_fits``)."""
+        leave half of ``memory_budget`` (bytes for the model and its cache; default: the GPU's memory) free
+        (``kernels.linear.packing_fits``)."""
         if dtype not in (torch.float32, torch.bfloat16):
             raise ValueError(f"dtype {dtype} is not supported (float32 or bfloat16)")
         self.layout, self.dtype, self.device = layout, dtype, torch.device(device)
         self.args, self.architecture = args, architecture
-        self.packed_weights = packed_weights
+        self.packed_weights, self.memory_budget = packed_weights, memory_budget
         self.parts = build_parts(layout)
         self.vocab_size = layout.vocab_size
         self.loaded = False
@@ -79,24 +81,26 @@ class Model:
     # ------------------------------------------------------------- build
     @classmethod
     def from_config(cls, config: Mapping[str, Any], dtype: torch.dtype, device: torch.device | str,
-                    packed_weights: Optional[bool] = None) -> "Model":
+                    packed_weights: Optional[bool] = None, memory_budget: Optional[int] = None) -> "Model":
         arch = get_architecture(config)
         args = arch.parse(config)
-        return cls(arch.layout(args), dtype, device, args=args, architecture=arch.name, packed_weights=packed_weights)
+        return cls(arch.layout(args), dtype, device, args=args, architecture=arch.name, packed_weights=packed_weights,
+                   memory_budget=memory_budget)
 
     @classmethod
     def from_folder(cls, model_dir: str | Path, dtype: torch.dtype, device: torch.device | str,
-                    packed_weights: Optional[bool] = None) -> "Model":
+                    packed_weights: Optional[bool] = None, memory_budget: Optional[int] = None) -> "Model":
         """The model that ``config.json`` names, with the folder's weights."""
-        model = cls.from_config(read_config_json(model_dir), dtype, device, packed_weights)
+        model = cls.from_config(read_config_json(model_dir), dtype, device, packed_weights, memory_budget)
         model.load(SafetensorsSource(model_dir))
         return model
 
     @classmethod
     def random(cls, config: Mapping[str, Any], seed: int, dtype: torch.dtype,
-               device: torch.device | str, packed_weights: Optional[bool] = None) -> "Model":
+               device: torch.device | str, packed_weights: Optional[bool] = None,
+               memory_budget: Optional[int] = None) -> "Model":
         """Seeded random weights drawn on the device, without a folder."""
-        model = cls.from_config(config, dtype, device, packed_weights)
+        model = cls.from_config(config, dtype, device, packed_weights, memory_budget)
         model.load(RandomSource(model.parts.tensor_specs(), seed, dtype, device))
         return model
 
@@ -106,7 +110,7 @@ class Model:
         pack = self.packed_weights
         if pack is None:
             matrix_bytes = sum(math.prod(s.shape) for s in specs if s.role == MATRIX) * 2
-            pack = self.dtype == torch.bfloat16 and packing_fits(matrix_bytes, self.device)
+            pack = self.dtype == torch.bfloat16 and packing_fits(matrix_bytes, self.device, self.memory_budget)
         with packing(pack and self.dtype == torch.bfloat16):
             for part in self.parts.all_parts:
                 tensors = {s.name: source.get(s.name) for s in part.tensor_specs()}

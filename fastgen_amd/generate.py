@@ -78,6 +78,14 @@ def cache_tokens_for_budget(model: Model, gen_args: GenArgs, bytes_per_token: in
     return -(-tokens // gen_args.cache_block) * gen_args.cache_block
 
 
+def memory_budget(gen_args: GenArgs) -> Optional[int]:
+    """The bytes that the weights and the cache share, where the arguments name them (``gpu_gb`` sizes the
+    cache): a model loaded for these arguments makes its second copy of the matrices
+    (``kernels.linear.StreamedMatrix``) only if that leaves half of the budget to the cache.  None: the
+    GPU's memory is the budget."""
+    return int(gen_args.gpu_gb * 1e9) if gen_args.max_seq < 0 and gen_args.gpu_gb > 0 else None
+
+
 class HfLoader:
     """A model folder in the Hugging Face layout: ``config.json``,
     ``model.safetensors`` (or shards with an index) and, optionally,
@@ -156,7 +164,7 @@ class Fastgen:
         device_ = torch.device(device)
         if device_.type != "cuda":
             raise RuntimeError("fastgen_amd runs on a GPU only")  # generate.py:148
-        model = Model.from_folder(model_dir, gen_args.dtype, device_)
+        model = Model.from_folder(model_dir, gen_args.dtype, device_, memory_budget=memory_budget(gen_args))
         if stop_tokens is None and isinstance(loader, HfLoader):
             tokenizer = loader.load_tokenizer()
             stop_tokens = tokenizer.stop_tokens if tokenizer is not None else None

@@ -105,16 +105,19 @@ def packing(on: bool):
         _pack_now = before
 
 
-def packing_fits(matrix_bytes: int, device) -> bool:
+def packing_fits(matrix_bytes: int, device, budget_bytes: Optional[int] = None) -> bool:
     """The rule for the second copy when nobody says otherwise (``FG_PACKED_WEIGHTS=0`` / ``1`` does): the
-    weights twice take at most half of the GPU's memory, so that at least half stays for the cache."""
+    weights twice take at most half of the memory that the model and its cache may use (``budget_bytes``;
+    default: all of the GPU's), so that at least half stays for the cache."""
     forced = os.environ.get("FG_PACKED_WEIGHTS", "")
     if forced in ("0", "1"):
         return forced == "1"
     dev = torch.device(device)
     if dev.type != "cuda":
         return False
-    return 2 * matrix_bytes <= torch.cuda.get_device_properties(dev).total_memory // 2
+    if budget_bytes is None:
+        budget_bytes = torch.cuda.get_device_properties(dev).total_memory
+    return 2 * matrix_bytes <= budget_bytes // 2
 
 
 def streamed(w: torch.Tensor) -> StreamedMatrix:

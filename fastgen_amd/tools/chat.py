@@ -56,7 +56,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     import json
 
     from ..engine import Model
-    from ..generate import Fastgen, GenArgs, Packet
+    from ..generate import Fastgen, GenArgs, Packet, memory_budget
     from .tokenizer import FolderTokenizer
 
     a = build_parser().parse_args(argv)
@@ -85,7 +85,8 @@ def main(argv: Optional[List[str]] = None) -> int:
                 config = json.load(f)
         else:
             config = read_config_json(a.model)
-        model = Model.random(config, a.random_weights, gen_args.dtype, "cuda:0")
+        budget = memory_budget(gen_args) if a.num_pages is None else None
+        model = Model.random(config, a.random_weights, gen_args.dtype, "cuda:0", memory_budget=budget)
         fg = Fastgen.from_model(model, gen_args, stop_tokens if stop_tokens is not None else (), a.num_pages)
     elif a.num_pages is not None:
         fg = Fastgen.from_model(Model.from_folder(a.model, gen_args.dtype, "cuda:0"), gen_args, stop_tokens, a.num_pages)

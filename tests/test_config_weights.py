@@ -197,6 +197,13 @@ def test_second_copy_of_the_matrices_is_a_matter_of_memory(monkeypatch):
 
     monkeypatch.delenv("FG_PACKED_WEIGHTS", raising=False)
     assert linear.packing_fits(1 << 30, "cpu") is False
+    import torch
+
+    monkeypatch.setattr(torch.cuda, "get_device_properties", lambda dev: type("P", (), {"total_memory": 288 << 30})())
+    assert linear.packing_fits(16 << 30, "cuda:0") is True  # 8B: 32 of 288 GB
+    assert linear.packing_fits(141 << 30, "cuda:0") is False  # 70B: one copy
+    assert linear.packing_fits(16 << 30, "cuda:0", budget_bytes=int(20e9)) is False  # a budget of 20 GB for both
+    assert linear.packing_fits(1 << 30, "cuda:0", budget_bytes=int(20e9)) is True
     monkeypatch.setenv("FG_PACKED_WEIGHTS", "1")
     assert linear.packing_fits(1 << 50, "cpu") is True
     monkeypatch.setenv("FG_PACKED_WEIGHTS", "0")
