@@ -115,7 +115,7 @@ def serve_workload(n_requests: int = 256, step_budget: int = 2048, shape: str = 
         "config": {"model": model_name, "requests": n_requests, "prompt_tokens": sum(plens),
                    "generated_tokens": sum(olens), "max_batch": max_batch, "step_budget": step_budget, "page_size": PAGE,
                    "engine_steps": engine.n_steps, "preemptions": engine.scheduler.n_preemptions,
-                   "weight_copies": 2 if engine.model.parts.head.weight.packed is not None else 1},
+                   "weight_copies": 2 if engine.model.packed() else 1},
     }), flush=True)
     return 0
 
@@ -175,7 +175,7 @@ def readme_workload(shape: str = "8b") -> int:
                    "max_batch": max_batch, "step_budget": 8192, "page_size": PAGE, "engine_steps": engine.n_steps,
                    "cache_tokens": pool, "cache": "free memory after the weights",
                    "preemptions": engine.scheduler.n_preemptions,
-                   "weight_copies": 2 if engine.model.parts.head.weight.packed is not None else 1,
+                   "weight_copies": 2 if engine.model.packed() else 1,
                    "published": published[1] if published else None},
     }), flush=True)
     return 0
@@ -290,7 +290,7 @@ def main() -> int:
             "hidden": D, "heads": H, "kv_heads": KV, "head_dim": hd, "ffn": F, "vocab": V, "page_size": PAGE,
             "rope_theta": cfg["rope_theta"], "rope_factor": cfg["rope_scaling"]["factor"], "norm_eps": cfg["rms_norm_eps"],
             # 2: every matrix is also held in the order the decode products read it (the roofline's bytes count one)
-            "weight_copies": 2 if model.parts.head.weight.packed is not None else 1,
+            "weight_copies": 2 if model.packed() else 1,
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",

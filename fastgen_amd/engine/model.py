@@ -139,6 +139,11 @@ class Model:
         """Whether every part's forward may be recorded into a HIP graph."""
         return all(getattr(p, "capturable", True) for p in self.parts.all_parts)
 
+    def packed(self) -> bool:
+        """Whether the matrices have their second copy in the streaming kernels' order."""
+        return any(isinstance(v, StreamedMatrix) and v.packed is not None
+                   for p in self.parts.all_parts for v in vars(p).values())
+
     def weight_bytes(self) -> int:
         seen, total = set(), 0
         for p in self.parts.all_parts:

@@ -152,8 +152,9 @@ class ModelRunner:
         self.graph_pool = None
         self.graph_capacity = graph_capacity_for  # batch size -> sequences of the recorded step that serves it
         self.max_graphs = 64
-        logger.info("weights %.2f GB; cache %s pages of %d tokens (%.2f GB), %d request slots; decode steps are %s",
-                    model.weight_bytes() / 1e9, pages, page_size,
+        logger.info("weights %.2f GB%s; cache %s pages of %d tokens (%.2f GB), %d request slots; decode steps are %s",
+                    model.weight_bytes() / 1e9, " (the matrices twice: rows and packed)" if model.packed() else "",
+                    pages, page_size,
                     sum(t.numel() * t.element_size() for t in self.storage.k + self.storage.v) / 1e9, max_requests,
                     "recorded as graphs" if self.use_graphs else "run eagerly")
         self.run_ahead = 16  # steps the host may prepare before the device has run them
