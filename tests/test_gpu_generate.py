@@ -406,6 +406,13 @@ def test_reference_style_interface(tiny_b):
     pool = fg2.engine.runner.cache.n_pages[0] * 64
     assert pool == pytest.approx((0.1e9 - fg2.engine.model.weight_bytes()) / per_token, abs=64)
     assert fg2.engine.scheduler.max_seq == 256  # one request is capped by max_position_embeddings
+    # the second copy of the matrices (in the streaming kernels' order) is made where the weights twice leave
+    # half of the budget to the cache: with 0.6 GB it is, with a budget of three times the weights it is not
+    assert fg2.engine.model.packed()
+    one_copy = fg2.engine.model.weight_bytes() / 2
+    fg3 = Fastgen.build(loader=loader, gen_args=GenArgs(gpu_gb=3 * one_copy / 1e9, prefill_gb=0,
+                                                        dtype=torch.bfloat16), tp_mesh=None, device="cuda:0")
+    assert not fg3.engine.model.packed() and fg3.engine.model.weight_bytes() < 1.1 * one_copy
 
 
 def test_command_line(tiny_b):
